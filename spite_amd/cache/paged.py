@@ -1,0 +1,187 @@
+"""The cache on the GPU: page pools per group of layers and per-request state tensors, with
+the host-side bookkeeping in the native cache manager.
+
+Layers are grouped by what they need: the same number of kv heads, head size and
+visibility (every key, the query's chunk, a window).  A group's pool is one tensor
+``[layers, 2, pages, kv_heads, page_size, head_dim]``; a page is the same row range in every
+layer of the group, so one block table serves all of them.
+"""
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..csrc import hostlib
+from ..parts.base import CacheNeed
+
+_KINDS = {"full": 0, "chunk": 1, "window": 2}
+
+
+class CacheError(RuntimeError):
+    pass
+
+
+class OutOfPages(CacheError):
+    pass
+
+
+@dataclass
+class Group:
+    key: tuple                   # (kv heads, head size, visibility, span)
+    cache_ids: List[int]
+    n_pages: int
+    kv: Optional[torch.Tensor]   # [layers, 2, pages, G, page_size, hd]
+
+
+class PagedCache:
+    def __init__(self, needs: Sequence[CacheNeed], page_size: int, num_pages, max_requests: int,
+                 dtype: torch.dtype, device, allocate: bool = True):
+        """``needs[i]``: what cache id i asks for.  ``num_pages``: pages of every group's pool
+        (an int), or one number per group in order of first use."""
+        self.page_size, self.max_requests, self.dtype, self.device = int(page_size), int(max_requests), dtype, device
+        self.groups: List[Group] = []
+        self._group_of: Dict[int, int] = {}
+        self._layer_in_group: Dict[int, int] = {}
+        by_key: Dict[tuple, int] = {}
+        for cid, need in enumerate(needs):
+            if need is None or need.kv is None:
+                continue
+            kv = need.kv
+            key = (kv.n_kv_heads, kv.head_dim, kv.visibility, kv.span if kv.visibility != "full" else 0)
+            if key not in by_key:
+                by_key[key] = len(self.groups)
+                self.groups.append(Group(key, [], 0, None))
+            g = by_key[key]
+            self._group_of[cid] = g
+            self._layer_in_group[cid] = len(self.groups[g].cache_ids)
+            self.groups[g].cache_ids.append(cid)
+        n_groups = len(self.groups)
+        pages = [int(num_pages)] * n_groups if isinstance(num_pages, int) else [int(x) for x in num_pages]
+        if len(pages) != n_groups:
+            raise CacheError(f"{len(pages)} pool sizes for {n_groups} groups")
+        for g, n in zip(self.groups, pages):
+            g.n_pages = n
+        lib = hostlib.lib()
+        kinds = hostlib.int_array(_KINDS[g.key[2]] for g in self.groups)
+        spans = hostlib.int_array(g.key[3] for g in self.groups)
+        npg = hostlib.int_array(pages)
+        self._h = lib.spc_create(self.page_size, self.max_requests, n_groups, kinds, spans, npg)
+        if not self._h:
+            raise CacheError(hostlib.last_error())
+        self._lib = lib
+        self.states: Dict[int, torch.Tensor] = {}
+        if allocate:
+            for g in self.groups:
+                G, hd = g.key[0], g.key[1]
+                g.kv = torch.zeros((len(g.cache_ids), 2, g.n_pages, G, self.page_size, hd), dtype=dtype, device=device)
+            for cid, need in enumerate(needs):
+                if need is not None and need.state is not None:
+                    self.states[cid] = torch.zeros((self.max_requests, *need.state.shape),
+                                                   dtype=need.state.dtype, device=device)
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            self._lib.spc_destroy(h)
+
+    # ------------------------------------------------------------------ bookkeeping
+    @property
+    def handle(self):
+        return self._h
+
+    def n_groups(self):
+        return len(self.groups)
+
+    def group_of(self, cache_id: int) -> int:
+        return self._group_of[cache_id]
+
+    def admit(self) -> int:
+        slot = self._lib.spc_admit(self._h)
+        if slot < 0:
+            raise CacheError(f"all {self.max_requests} request slots are taken")
+        self.zero_state(slot)
+        return slot
+
+    def zero_state(self, slot: int):
+        for st in self.states.values():
+            st[slot].zero_()
+
+    def live(self, slot):
+        return bool(self._lib.spc_live(self._h, slot))
+
+    def cached(self, slot) -> int:
+        return int(self._lib.spc_cached(self._h, slot))
+
+    def can_reserve(self, slot, n) -> bool:
+        return bool(self._lib.spc_can_reserve(self._h, slot, n))
+
+    def reserve(self, slot, n):
+        rc = self._lib.spc_reserve(self._h, slot, n)
+        if rc == -1:
+            raise OutOfPages(f"no pages for {n} more positions of slot {slot}: free "
+                             f"{[self.free_pages(g) for g in range(self.n_groups())]}")
+        if rc != 0:
+            raise CacheError(f"reserve: slot {slot} is not live")
+
+    def commit(self, slot, n):
+        rc = self._lib.spc_commit(self._h, slot, n)
+        if rc != 0:
+            raise CacheError(f"commit({slot}, {n}) failed with {rc}: not live, or more than was reserved")
+
+    def release(self, slot):
+        if self._lib.spc_release(self._h, slot) != 0:
+            raise CacheError(f"release: slot {slot} is not live")
+
+    def free_pages(self, g) -> int:
+        return int(self._lib.spc_free_pages(self._h, g))
+
+    def total_pages(self, g) -> int:
+        return int(self._lib.spc_total_pages(self._h, g))
+
+    def free_slots(self) -> int:
+        return int(self._lib.spc_free_slots(self._h))
+
+    def peak_pages(self, total, portion, g) -> int:
+        return int(self._lib.spc_peak_pages(self._h, total, portion, g))
+
+    def block_table(self, slot, g) -> List[int]:
+        n = self._lib.spc_table_len(self._h, slot, g)
+        if n < 0:
+            raise CacheError(f"slot {slot} is not live")
+        buf = (ctypes.c_int * max(n, 1))()
+        self._lib.spc_table(self._h, slot, g, buf, n)
+        return list(buf[:n])
+
+    def check(self):
+        if self._lib.spc_check(self._h) != 0:
+            raise CacheError(hostlib.last_error())
+
+    # ------------------------------------------------------------------ step metadata
+    def fill_step(self, slots, starts, counts, g, slot_map_out: np.ndarray, table_out: np.ndarray):
+        """Cache rows of every token of the step and one block-table row per entry."""
+        off = 0
+        width = table_out.shape[1]
+        for i, (s, st, n) in enumerate(zip(slots, starts, counts)):
+            s, st, n = int(s), int(st), int(n)
+            if self._lib.spc_slot_mapping(self._h, s, g, st, n, slot_map_out[off:off + n].ctypes.data) != 0:
+                raise CacheError(f"slot {s} is not live")
+            tl = self._lib.spc_table_len(self._h, s, g)
+            if tl > width:
+                raise CacheError("block table wider than planned")
+            row = table_out[i]
+            row[tl:] = -1
+            if tl:
+                self._lib.spc_table(self._h, s, g, row.ctypes.data_as(ctypes.POINTER(ctypes.c_int)), tl)
+            off += n
+
+    def table_len(self, slot, g) -> int:
+        return int(self._lib.spc_table_len(self._h, slot, g))
+
+    def layer_pages(self, cache_id: int):
+        g = self.groups[self._group_of[cache_id]]
+        li = self._layer_in_group[cache_id]
+        return g.kv[li, 0], g.kv[li, 1]

@@ -1,0 +1,287 @@
+// Row-wise kernels of the step: embedding gather, residual add + RMSNorm, rotation /
+// qk-norm / temperature + cache write, top-1 router and the expert plan.
+// One workgroup per row (or per token and head); all reductions in fp32 in an order that
+// depends on the row's width only, never on what else is in the batch.
+#include "common.h"
+
+static thread_local char g_err[512];
+int sp_fail(const char* fmt, ...) {
+    va_list ap; va_start(ap, fmt); vsnprintf(g_err, sizeof g_err, fmt, ap); va_end(ap);
+    return -1;
+}
+extern "C" const char* spite_hip_last_error() { return g_err; }
+extern "C" int spite_hip_abi_version() { return 1; }
+
+// ------------------------------------------------------------------ embedding
+template <typename T>
+__global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table,
+                             float* __restrict__ h, int d, int vocab) {
+    const int t = blockIdx.x;
+    const int id = ids[t];
+    const bool ok = id >= 0 && id < vocab;
+    const T* row = table + (size_t)(ok ? id : 0) * d;
+    for (int c = threadIdx.x; c < d; c += blockDim.x)
+        h[(size_t)t * d + c] = ok ? to_f32<T>(row[c]) : 0.f;
+}
+
+extern "C" int spite_embed(const int* ids, const void* table, int dtype, float* h, int T, int d,
+                           int vocab, hipStream_t st) {
+    SP_REQUIRE(T >= 0 && d > 0 && vocab > 0, "embed: bad sizes T=%d d=%d vocab=%d", T, d, vocab);
+    if (T == 0) return 0;
+    if (dtype == SP_F32) embed_kernel<float><<<T, 256, 0, st>>>(ids, (const float*)table, h, d, vocab);
+    else if (dtype == SP_BF16) embed_kernel<bf16><<<T, 256, 0, st>>>(ids, (const bf16*)table, h, d, vocab);
+    else return sp_fail("embed: unknown dtype %d", dtype);
+    SP_LAUNCH_CHECK("embed");
+    return 0;
+}
+
+// ------------------------------------------------------------------ residual add + RMSNorm
+// v = h[r] + d1[r] + d2[r]; (h[r] = v); out[i] = v * 1/sqrt(mean(v^2)+eps) * w, r = rows ? rows[i] : i.
+template <typename TO>
+__global__ void add_rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ d1,
+                                   const float* __restrict__ d2, const float* __restrict__ w,
+                                   TO* __restrict__ out, float* __restrict__ out32,
+                                   const int* __restrict__ rows, int d, float eps, int write_h) {
+    __shared__ float red[4];
+    const int i = blockIdx.x;
+    const size_t r = rows ? (size_t)rows[i] : (size_t)i;
+    float* hr = h + r * d;
+    const float* a = d1 ? d1 + r * d : nullptr;
+    const float* b = d2 ? d2 + r * d : nullptr;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < d; c += 256) {
+        float v = hr[c];
+        if (a) v += a[c];
+        if (b) v += b[c];
+        if (write_h) hr[c] = v;
+        ss += v * v;
+    }
+    const float ms = block_sum<256>(ss, red) / (float)d;
+    const float scale = 1.0f / sqrtf(ms + eps);
+    for (int c = threadIdx.x; c < d; c += 256) {
+        float v = hr[c];
+        if (!write_h) { if (a) v += a[c]; if (b) v += b[c]; }
+        const float y = v * scale * w[c];
+        if (out) out[(size_t)i * d + c] = from_f32<TO>(y);
+        if (out32) out32[(size_t)i * d + c] = y;
+    }
+}
+
+extern "C" int spite_add_rmsnorm(float* h, const float* d1, const float* d2, const float* w, void* out,
+                                 int out_dtype, float* out32, const int* rows, int n_rows, int d,
+                                 float eps, int write_h, hipStream_t st) {
+    SP_REQUIRE(n_rows >= 0 && d > 0 && eps > 0.f, "add_rmsnorm: bad sizes rows=%d d=%d eps=%g", n_rows, d, eps);
+    if (n_rows == 0) return 0;
+    if (out_dtype == SP_F32)
+        add_rmsnorm_kernel<float><<<n_rows, 256, 0, st>>>(h, d1, d2, w, (float*)out, out32, rows, d, eps, write_h);
+    else if (out_dtype == SP_BF16)
+        add_rmsnorm_kernel<bf16><<<n_rows, 256, 0, st>>>(h, d1, d2, w, (bf16*)out, out32, rows, d, eps, write_h);
+    else return sp_fail("add_rmsnorm: unknown dtype %d", out_dtype);
+    SP_LAUNCH_CHECK("add_rmsnorm");
+    return 0;
+}
+
+// ------------------------------------------------------------------ rotation, qk-norm, temperature, cache write
+// One wave per (token, head).  Heads [0,H) are queries, [H,H+G) keys, [H+G,H+2G) values of
+// the fused projection row.  Queries and keys: rotate by pos*inv_freq (if use_rope), then
+// the weightless RMS norm over the head (if use_norm); queries alone are then multiplied by
+// ln(floor((pos+1)/floor_scale)+1)*attn_scale+1 (if use_temp).  Keys and values go to the
+// request's page: cache row = slot_map[t] = page*page_size + offset, pages laid out
+// [page][kv head][offset][hd].
+#define SP_MAX_PAIRS 4   // head sizes up to 512
+template <typename T>
+__global__ void rope_kvwrite_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
+                                    T* __restrict__ k_pages, T* __restrict__ v_pages,
+                                    const int* __restrict__ positions, const int* __restrict__ slot_map,
+                                    const float* __restrict__ inv_freq, int H, int G, int hd, int ps,
+                                    int use_rope, int adjacent, int use_norm, float norm_eps,
+                                    int use_temp, int floor_scale, float attn_scale) {
+    const int t = blockIdx.x;
+    const int hh = blockIdx.y;
+    const int lane = threadIdx.x;
+    const int half = hd >> 1;
+    const int row_w = (H + 2 * G) * hd;
+    const T* src = qkv + (size_t)t * row_w + (size_t)hh * hd;
+    const int pos = positions[t];
+    const bool is_q = hh < H;
+    const bool is_v = hh >= H + G;
+
+    T* dst;
+    if (is_q) {
+        dst = q_out + ((size_t)t * H + hh) * hd;
+    } else {
+        const int slot = slot_map[t];
+        if (slot < 0) return;
+        const int g = is_v ? hh - H - G : hh - H;
+        const size_t page = slot / ps, off = slot % ps;
+        dst = (is_v ? v_pages : k_pages) + ((page * G + g) * ps + off) * hd;
+    }
+    if (is_v) {
+        for (int c = lane; c < hd; c += 64) dst[c] = src[c];
+        return;
+    }
+    float x0[SP_MAX_PAIRS], x1[SP_MAX_PAIRS];
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < SP_MAX_PAIRS; ++u) {
+        const int i = lane + u * 64;
+        if (i < half) {
+            const int i0 = adjacent ? 2 * i : i;
+            const int i1 = adjacent ? 2 * i + 1 : i + half;
+            float a = to_f32<T>(src[i0]), b = to_f32<T>(src[i1]);
+            if (use_rope) {
+                const float ang = (float)pos * inv_freq[i];
+                float sn, cs;
+                sincosf(ang, &sn, &cs);
+                const float ra = a * cs - b * sn;
+                const float rb = a * sn + b * cs;
+                a = ra; b = rb;
+            }
+            x0[u] = a; x1[u] = b;
+            ss += a * a + b * b;
+        }
+    }
+    float scale = 1.f;
+    if (use_norm) {
+        ss = wave_sum(ss);
+        scale = 1.0f / sqrtf(ss / (float)hd + norm_eps);
+    }
+    if (is_q && use_temp) {
+        const int k = (pos + 1) / floor_scale;
+        scale *= logf((float)k + 1.0f) * attn_scale + 1.0f;
+    }
+#pragma unroll
+    for (int u = 0; u < SP_MAX_PAIRS; ++u) {
+        const int i = lane + u * 64;
+        if (i < half) {
+            const int i0 = adjacent ? 2 * i : i;
+            const int i1 = adjacent ? 2 * i + 1 : i + half;
+            dst[i0] = from_f32<T>(x0[u] * scale);
+            dst[i1] = from_f32<T>(x1[u] * scale);
+        }
+    }
+}
+
+extern "C" int spite_rope_kvwrite(const void* qkv, void* q_out, void* k_pages, void* v_pages, int dtype,
+                                  const int* positions, const int* slot_map, const float* inv_freq,
+                                  int T, int H, int G, int hd, int page_size, int use_rope, int adjacent,
+                                  int use_norm, float norm_eps, int use_temp, int floor_scale,
+                                  float attn_scale, int write_kv, hipStream_t st) {
+    SP_REQUIRE(T >= 0 && H > 0 && G > 0 && hd > 0 && page_size > 0, "rope_kvwrite: bad sizes");
+    SP_REQUIRE(hd % 2 == 0 && hd <= 128 * SP_MAX_PAIRS, "rope_kvwrite: head size %d must be even and <= %d",
+               hd, 128 * SP_MAX_PAIRS);
+    SP_REQUIRE(!use_temp || floor_scale > 0, "rope_kvwrite: floor_scale %d must be >= 1", floor_scale);
+    SP_REQUIRE(!use_rope || inv_freq, "rope_kvwrite: rotation needs a frequency table");
+    SP_REQUIRE(H + 2 * G <= 65535, "rope_kvwrite: too many heads");
+    if (T == 0) return 0;
+    dim3 grid(T, write_kv ? H + 2 * G : H);
+    if (dtype == SP_F32)
+        rope_kvwrite_kernel<float><<<grid, 64, 0, st>>>((const float*)qkv, (float*)q_out, (float*)k_pages,
+            (float*)v_pages, positions, slot_map, inv_freq, H, G, hd, page_size, use_rope, adjacent, use_norm,
+            norm_eps, use_temp, floor_scale, attn_scale);
+    else if (dtype == SP_BF16)
+        rope_kvwrite_kernel<bf16><<<grid, 64, 0, st>>>((const bf16*)qkv, (bf16*)q_out, (bf16*)k_pages,
+            (bf16*)v_pages, positions, slot_map, inv_freq, H, G, hd, page_size, use_rope, adjacent, use_norm,
+            norm_eps, use_temp, floor_scale, attn_scale);
+    else return sp_fail("rope_kvwrite: unknown dtype %d", dtype);
+    SP_LAUNCH_CHECK("rope_kvwrite");
+    return 0;
+}
+
+// ------------------------------------------------------------------ top-1 sigmoid router
+// One wave per token: logits = W_r . x in fp32, the largest logit wins and the lowest index
+// wins a tie, weight = 1/(1+exp(-logit)).
+__global__ void router_top1_kernel(const float* __restrict__ x, const float* __restrict__ wr,
+                                   int* __restrict__ expert, float* __restrict__ weight,
+                                   float* __restrict__ logits_out, int d, int E) {
+    const int t = blockIdx.x;
+    const int lane = threadIdx.x;
+    const float* xr = x + (size_t)t * d;
+    float best = 0.f; int best_e = -1;
+    for (int e = 0; e < E; ++e) {
+        const float* w = wr + (size_t)e * d;
+        float acc = 0.f;
+        for (int c = lane; c < d; c += 64) acc += w[c] * xr[c];
+        acc = wave_sum(acc);
+        if (logits_out && lane == 0) logits_out[(size_t)t * E + e] = acc;
+        if (best_e < 0 || acc > best) { best = acc; best_e = e; }
+    }
+    if (lane == 0) {
+        expert[t] = best_e;
+        weight[t] = 1.0f / (1.0f + expf(-best));
+    }
+}
+
+extern "C" int spite_router_top1(const float* x, const float* wr, int* expert, float* weight,
+                                 float* logits_out, int T, int d, int E, hipStream_t st) {
+    SP_REQUIRE(T >= 0 && d > 0 && E > 0, "router: bad sizes T=%d d=%d E=%d", T, d, E);
+    if (T == 0) return 0;
+    router_top1_kernel<<<T, 64, 0, st>>>(x, wr, expert, weight, logits_out, d, E);
+    SP_LAUNCH_CHECK("router_top1");
+    return 0;
+}
+
+// ------------------------------------------------------------------ expert plan
+// From expert[t], weight[t] build the row list that the grouped products walk:
+//   slots [0,T): tokens in order of expert (stable), src[s] = token, scale[s] = its weight,
+//                dst[s] = token;
+//   slots [T,2T) (if shared): src = dst-T = token, scale 1, dst[s] = T + token  (the group E
+//                that every token visits);
+//   offsets[g] = first slot of group g, g in [0, E+1] (+1 with the shared group).
+// Each thread ranks one token by counting over all tokens in shared memory: no atomics, the
+// order is the same on every run.
+__global__ void moe_plan_kernel(const int* __restrict__ expert, const float* __restrict__ weight,
+                                int* __restrict__ src, float* __restrict__ scale, int* __restrict__ dst,
+                                int* __restrict__ offsets, int T, int E, int shared) {
+    extern __shared__ unsigned short e_of[];
+    for (int i = threadIdx.x; i < T; i += blockDim.x) e_of[i] = (unsigned short)expert[i];
+    __syncthreads();
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t < T) {
+        const int me = e_of[t];
+        int rank = 0;
+        for (int j = 0; j < T; ++j) {
+            const int ej = e_of[j];
+            rank += (ej < me) || (ej == me && j < t);
+        }
+        src[rank] = t; scale[rank] = weight[t]; dst[rank] = t;
+        if (shared) { src[T + t] = t; scale[T + t] = 1.0f; dst[T + t] = T + t; }
+    }
+    if (blockIdx.x == 0) {
+        for (int g = threadIdx.x; g <= E; g += blockDim.x) {
+            int c = 0;
+            for (int j = 0; j < T; ++j) c += e_of[j] < g;
+            offsets[g] = c;
+        }
+        if (shared && threadIdx.x == 0) offsets[E + 1] = 2 * T;
+    }
+}
+
+extern "C" int spite_moe_plan(const int* expert, const float* weight, int* src, float* scale, int* dst,
+                              int* offsets, int T, int E, int shared, hipStream_t st) {
+    SP_REQUIRE(T >= 0 && E > 0 && E < 65535, "moe_plan: bad sizes T=%d E=%d", T, E);
+    SP_REQUIRE(T <= 32768, "moe_plan: %d tokens in one step, at most 32768", T);
+    const int grid = T > 0 ? (T + 255) / 256 : 1;
+    moe_plan_kernel<<<grid, 256, (size_t)(T > 0 ? T : 1) * sizeof(unsigned short), st>>>(
+        expert, weight, src, scale, dst, offsets, T, E, shared);
+    SP_LAUNCH_CHECK("moe_plan");
+    return 0;
+}
+
+// ------------------------------------------------------------------ small helpers
+template <typename TI, typename TO>
+__global__ void convert_kernel(const TI* __restrict__ in, TO* __restrict__ out, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        out[i] = from_f32<TO>(to_f32<TI>(in[i]));
+}
+extern "C" int spite_convert(const void* in, int in_dtype, void* out, int out_dtype, size_t n, hipStream_t st) {
+    if (n == 0) return 0;
+    const int grid = (int)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
+    if (in_dtype == SP_F32 && out_dtype == SP_BF16) convert_kernel<float, bf16><<<grid, 256, 0, st>>>((const float*)in, (bf16*)out, n);
+    else if (in_dtype == SP_BF16 && out_dtype == SP_F32) convert_kernel<bf16, float><<<grid, 256, 0, st>>>((const bf16*)in, (float*)out, n);
+    else if (in_dtype == SP_F32 && out_dtype == SP_F32) convert_kernel<float, float><<<grid, 256, 0, st>>>((const float*)in, (float*)out, n);
+    else if (in_dtype == SP_BF16 && out_dtype == SP_BF16) convert_kernel<bf16, bf16><<<grid, 256, 0, st>>>((const bf16*)in, (bf16*)out, n);
+    else return sp_fail("convert: unknown dtypes %d -> %d", in_dtype, out_dtype);
+    SP_LAUNCH_CHECK("convert");
+    return 0;
+}

@@ -1,0 +1,235 @@
+"""ctypes binding of the gfx950 kernel library: one Python function per entry point.
+
+Arguments are torch tensors on the GPU; each wrapper checks device, dtype, contiguity and the
+shapes that the kernel's indexing assumes before it launches, and raises ``KernelError`` with
+the library's message when the library refuses a size.  There is no fallback: without the
+library, or with a tensor that is not on the GPU, the call fails.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_int, c_long, c_float, c_void_p, c_size_t, c_char_p
+
+import torch
+
+from . import build
+
+F32, BF16 = 0, 1
+VIS = {"full": 0, "chunk": 1, "window": 2}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        l = build.load("hip")
+        l.spite_hip_last_error.restype = c_char_p
+        P, I, L, F = c_void_p, c_int, c_long, c_float
+        sigs = {
+            "spite_embed": [P, P, I, P, I, I, I, P],
+            "spite_add_rmsnorm": [P, P, P, P, P, I, P, P, I, I, F, I, P],
+            "spite_rope_kvwrite": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, I, I, F, I, P],
+            "spite_router_top1": [P, P, P, P, P, I, I, I, P],
+            "spite_moe_plan": [P, P, P, P, P, P, I, I, I, P],
+            "spite_convert": [P, I, P, I, c_size_t, P],
+            "spite_gemm_generic": [P, I, P, L, I, P, I, I, I, I, I, P, I, P, P, P, I, P],
+            "spite_attn_generic": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, P],
+            "spite_sample_rows": [P, I, I, I, P, P, P, P],
+        }
+        for name, args in sigs.items():
+            fn = getattr(l, name)
+            fn.argtypes = args
+            fn.restype = c_int
+        _lib = l
+    return _lib
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    if dt == torch.float32:
+        return F32
+    if dt == torch.bfloat16:
+        return BF16
+    raise KernelError(f"no kernel for dtype {dt}; the engine computes in float32 or bfloat16")
+
+
+def _ptr(t, name, dtype=None, optional=False):
+    if t is None:
+        if optional:
+            return None
+        raise KernelError(f"{name}: missing tensor")
+    if not t.is_cuda:
+        raise KernelError(f"{name}: tensor is on {t.device}; the kernels run on the GPU only")
+    if not t.is_contiguous():
+        raise KernelError(f"{name}: tensor is not contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name}: dtype {t.dtype}, expected {dtype}")
+    return t.data_ptr()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _check(rc, what):
+    if rc != 0:
+        raise KernelError(f"{what}: {lib().spite_hip_last_error().decode()}")
+
+
+# --------------------------------------------------------------------------------------------
+def embed(ids, table, h):
+    """h[t,:] = table[ids[t],:] as fp32.  ids int32 [T], table [V,d], h fp32 [T,d]."""
+    T, d = h.shape
+    if ids.numel() != T or table.shape[1] != d:
+        raise KernelError(f"embed: ids {tuple(ids.shape)}, table {tuple(table.shape)}, h {tuple(h.shape)}")
+    _check(lib().spite_embed(_ptr(ids, "ids", torch.int32), _ptr(table, "table"), dtype_code(table.dtype),
+                             _ptr(h, "h", torch.float32), T, d, table.shape[0], _stream()), "embed")
+
+
+def add_rmsnorm(h, w, eps, out=None, out32=None, d1=None, d2=None, rows=None, n_rows=None, write_h=True):
+    """v = h[r] + d1[r] + d2[r] (stored back if write_h); out[i] = rmsnorm(v) * w with r =
+    rows[i] or i.  h, d1, d2, out32 fp32; w fp32 [d]; out fp32 or bf16."""
+    d = h.shape[-1]
+    n = n_rows if n_rows is not None else (rows.numel() if rows is not None else h.shape[0])
+    for name, t in (("d1", d1), ("d2", d2)):
+        if t is not None and (t.shape[-1] != d or t.shape[0] < h.shape[0]):
+            raise KernelError(f"add_rmsnorm: {name} {tuple(t.shape)} does not match h {tuple(h.shape)}")
+    if w.numel() != d:
+        raise KernelError(f"add_rmsnorm: weight of {w.numel()} for rows of {d}")
+    for name, t in (("out", out), ("out32", out32)):
+        if t is not None and (t.shape[-1] != d or t.shape[0] < n):
+            raise KernelError(f"add_rmsnorm: {name} {tuple(t.shape)} is too small for {n} rows of {d}")
+    if rows is None and n > h.shape[0]:
+        raise KernelError("add_rmsnorm: more rows asked than h holds")
+    _check(lib().spite_add_rmsnorm(
+        _ptr(h, "h", torch.float32), _ptr(d1, "d1", torch.float32, True), _ptr(d2, "d2", torch.float32, True),
+        _ptr(w, "w", torch.float32), _ptr(out, "out", None, True),
+        dtype_code(out.dtype) if out is not None else F32, _ptr(out32, "out32", torch.float32, True),
+        _ptr(rows, "rows", torch.int32, True), n, d, float(eps), int(write_h), _stream()), "add_rmsnorm")
+
+
+def rope_kvwrite(qkv, q_out, k_pages, v_pages, positions, slot_map, inv_freq, H, G, hd, page_size, *,
+                 use_rope, adjacent, use_norm, norm_eps, use_temp, floor_scale, attn_scale, write_kv=True):
+    """Rotation, weightless qk-norm and temperature of the fused projection's rows; keys and
+    values go to their cache rows.  qkv [T,(H+2G)*hd]; q_out [T,H*hd]; pages
+    [n_pages, G, page_size, hd]."""
+    T = qkv.shape[0]
+    if qkv.shape[1] != (H + 2 * G) * hd:
+        raise KernelError(f"rope_kvwrite: qkv {tuple(qkv.shape)} for H={H} G={G} hd={hd}")
+    if q_out.numel() < T * H * hd or positions.numel() < T:
+        raise KernelError("rope_kvwrite: q_out or positions too small")
+    if write_kv:
+        if slot_map.numel() < T:
+            raise KernelError("rope_kvwrite: slot map too small")
+        if tuple(k_pages.shape[1:]) != (G, page_size, hd) or k_pages.shape != v_pages.shape:
+            raise KernelError(f"rope_kvwrite: pages {tuple(k_pages.shape)} for G={G} page={page_size} hd={hd}")
+    if use_rope and inv_freq.numel() != hd // 2:
+        raise KernelError("rope_kvwrite: frequency table does not match the head size")
+    dt = qkv.dtype
+    _check(lib().spite_rope_kvwrite(
+        _ptr(qkv, "qkv"), _ptr(q_out, "q_out", dt), _ptr(k_pages, "k_pages", dt, not write_kv),
+        _ptr(v_pages, "v_pages", dt, not write_kv), dtype_code(dt), _ptr(positions, "positions", torch.int32),
+        _ptr(slot_map, "slot_map", torch.int32, not write_kv), _ptr(inv_freq, "inv_freq", torch.float32, not use_rope),
+        T, H, G, hd, page_size, int(use_rope), int(adjacent), int(use_norm), float(norm_eps), int(use_temp),
+        int(floor_scale), float(attn_scale), int(write_kv), _stream()), "rope_kvwrite")
+
+
+def router_top1(x32, w_router, expert, weight, logits_out=None):
+    """Top-1 sigmoid router on fp32 rows.  x32 [T,d], w_router fp32 [E,d]."""
+    T, d = x32.shape
+    E = w_router.shape[0]
+    if w_router.shape[1] != d or expert.numel() < T or weight.numel() < T:
+        raise KernelError("router_top1: shapes do not match")
+    if logits_out is not None and logits_out.numel() < T * E:
+        raise KernelError("router_top1: logits_out too small")
+    _check(lib().spite_router_top1(_ptr(x32, "x32", torch.float32), _ptr(w_router, "w_router", torch.float32),
+                                   _ptr(expert, "expert", torch.int32), _ptr(weight, "weight", torch.float32),
+                                   _ptr(logits_out, "logits_out", torch.float32, True), T, d, E, _stream()),
+           "router_top1")
+
+
+def moe_plan(expert, weight, src, scale, dst, offsets, T, E, shared):
+    """Row list of the grouped products from the router's choice (see the kernel)."""
+    n = 2 * T if shared else T
+    if src.numel() < n or scale.numel() < n or dst.numel() < n or offsets.numel() < E + 1 + int(bool(shared)):
+        raise KernelError("moe_plan: output arrays too small")
+    if expert.numel() < T or weight.numel() < T:
+        raise KernelError("moe_plan: inputs too small")
+    _check(lib().spite_moe_plan(_ptr(expert, "expert", torch.int32), _ptr(weight, "weight", torch.float32),
+                                _ptr(src, "src", torch.int32), _ptr(scale, "scale", torch.float32),
+                                _ptr(dst, "dst", torch.int32), _ptr(offsets, "offsets", torch.int32),
+                                T, E, int(bool(shared)), _stream()), "moe_plan")
+
+
+def convert(src, dst):
+    if src.numel() != dst.numel():
+        raise KernelError("convert: sizes differ")
+    _check(lib().spite_convert(_ptr(src, "src"), dtype_code(src.dtype), _ptr(dst, "dst"), dtype_code(dst.dtype),
+                               src.numel(), _stream()), "convert")
+
+
+def gemm_generic(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None,
+                 glu=False):
+    """Y = A . W^T (see gemm_generic.hip).  a [rows,K]; w [groups, N or 2N, K] or [N or 2N, K];
+    y [rows,N]."""
+    if a.shape[-1] != K or y.shape[-1] != N:
+        raise KernelError(f"gemm: a {tuple(a.shape)}, y {tuple(y.shape)} for N={N} K={K}")
+    rows_w = 2 * N if glu else N
+    if w.shape[-1] != K or w.shape[-2] != rows_w:
+        raise KernelError(f"gemm: weight {tuple(w.shape)} for N={N} K={K} glu={glu}")
+    groups_w = w.shape[0] if w.dim() == 3 else 1
+    if offsets is not None:
+        if groups_w < n_groups or offsets.numel() < n_groups + 1:
+            raise KernelError("gemm: fewer weight groups or offsets than groups")
+    if a_rows is None and a.shape[0] < M:
+        raise KernelError("gemm: A has fewer rows than M")
+    if y_rows is None and y.shape[0] < M:
+        raise KernelError("gemm: Y has fewer rows than M")
+    for name, t in (("a_rows", a_rows), ("a_scale", a_scale), ("y_rows", y_rows)):
+        if t is not None and t.numel() < M:
+            raise KernelError(f"gemm: {name} shorter than M")
+    if w.dtype != a.dtype:
+        raise KernelError(f"gemm: activations {a.dtype} against weights {w.dtype}")
+    _check(lib().spite_gemm_generic(
+        _ptr(a, "a"), a.stride(0) if a.dim() == 2 else K, _ptr(w, "w"), rows_w * K, dtype_code(a.dtype),
+        _ptr(y, "y"), dtype_code(y.dtype), y.stride(0), M, N, K, _ptr(offsets, "offsets", torch.int32, True), n_groups,
+        _ptr(a_rows, "a_rows", torch.int32, True), _ptr(a_scale, "a_scale", torch.float32, True),
+        _ptr(y_rows, "y_rows", torch.int32, True), int(glu), _stream()), "gemm")
+
+
+def attn_generic(q, k_pages, v_pages, out, positions, seq_of_token, block_table, T, H, G, hd, page_size,
+                 vis, span, scale):
+    """Attention over the paged cache, any mix of portions and single tokens.  q/out
+    [T,H*hd]; block_table int32 [n_seqs, max_blocks]."""
+    if q.numel() < T * H * hd or out.numel() < T * H * hd:
+        raise KernelError("attention: q or out too small")
+    if tuple(k_pages.shape[1:]) != (G, page_size, hd) or k_pages.shape != v_pages.shape:
+        raise KernelError(f"attention: pages {tuple(k_pages.shape)} for G={G} page={page_size} hd={hd}")
+    if block_table.dim() != 2 or positions.numel() < T or seq_of_token.numel() < T:
+        raise KernelError("attention: metadata too small")
+    dt = q.dtype
+    _check(lib().spite_attn_generic(
+        _ptr(q, "q"), _ptr(k_pages, "k_pages", dt), _ptr(v_pages, "v_pages", dt), _ptr(out, "out", dt),
+        dtype_code(dt), _ptr(positions, "positions", torch.int32), _ptr(seq_of_token, "seq_of_token", torch.int32),
+        _ptr(block_table, "block_table", torch.int32), block_table.shape[1], T, H, G, hd, page_size,
+        VIS[vis], int(span or 0), float(scale), _stream()), "attention")
+
+
+def sample_rows(logits, temperature, uniform, out, n_rows=None):
+    """out[r] = arg-max of row r (temperature[r] <= 0 or no temperatures) or the inverse-CDF
+    draw with uniform[r].  logits fp32 [n,V]."""
+    n = n_rows if n_rows is not None else logits.shape[0]
+    if out.numel() < n or logits.shape[0] < n:
+        raise KernelError("sample: too few rows")
+    for name, t in (("temperature", temperature), ("uniform", uniform)):
+        if t is not None and t.numel() < n:
+            raise KernelError(f"sample: {name} shorter than the rows")
+    _check(lib().spite_sample_rows(_ptr(logits, "logits", torch.float32), logits.stride(0), n, logits.shape[1],
+                                   _ptr(temperature, "temperature", torch.float32, True),
+                                   _ptr(uniform, "uniform", torch.float32, True),
+                                   _ptr(out, "out", torch.int32), _stream()), "sample")

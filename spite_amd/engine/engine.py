@@ -1,0 +1,271 @@
+"""The engine: a model on the GPU, its cache, and the one step function.
+
+``Engine.step(entries)`` takes a batch of (request slot, its next tokens, wanted logit
+places): portions of prompts beside single decoded tokens, cut anywhere.  It runs only the
+tokens it is given, as one batch, against what earlier steps left in the cache, and returns
+fp32 logits at the wanted places.  The reference's ``forward(tokens, logits_out, ctx)``
+(crates/spite-models/src/lib.rs:330-335) is the one-request, every-position special case.
+"""
+from __future__ import annotations
+
+import json
+import os
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Union
+
+import numpy as np
+import torch
+
+from ..cache.paged import PagedCache, CacheError, OutOfPages
+from ..config import read_config
+from ..csrc import hipops
+from ..parts.base import ModelSpec, LayerCall
+from ..weights.loader import load_weights
+from .context import Env, Workspace, StepContext, LayerCache, HostBatch
+from .model import Model
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
+           "f32": torch.float32}
+_CKPT_DTYPES = {"bfloat16": torch.bfloat16, "float16": torch.float16, "float32": torch.float32}
+
+
+class EngineError(RuntimeError):
+    pass
+
+
+@dataclass
+class StepEntry:
+    slot: int
+    tokens: Sequence[int]
+    want: Sequence[int] = ()        # places among ``tokens`` whose logits are asked for
+
+
+class StepMeta:
+    """Metadata of one step: built on the host, sent to the GPU in one copy."""
+
+    def __init__(self, engine: "Engine", entries: Sequence[StepEntry]):
+        cache = engine.cache
+        n = len(entries)
+        slots = np.array([e.slot for e in entries], dtype=np.int32)
+        counts = np.array([len(e.tokens) for e in entries], dtype=np.int32)
+        starts = np.array([cache.cached(int(s)) for s in slots], dtype=np.int32)
+        cu = np.zeros(n + 1, dtype=np.int32)
+        np.cumsum(counts, out=cu[1:])
+        T = int(cu[-1])
+        n_groups = cache.n_groups()
+        widths = []
+        for g in range(n_groups):
+            w = max([cache.table_len(int(s), g) for s in slots], default=1)
+            widths.append(max(4, (w + 3) // 4 * 4))
+        rows = []
+        for i, e in enumerate(entries):
+            for w in e.want:
+                if not 0 <= int(w) < counts[i]:
+                    raise EngineError(f"entry {i}: wanted place {w} outside its {counts[i]} tokens")
+                rows.append(int(cu[i]) + int(w))
+        n_out = len(rows)
+        # layout of the one int32 buffer
+        sizes = [("token_ids", T), ("positions", T), ("seq_of_token", T), ("cu_seqlens", n + 1),
+                 ("seq_slots", n), ("seq_starts", n), ("logit_rows", n_out)]
+        for g in range(n_groups):
+            sizes += [(f"slot_map{g}", T), (f"table{g}", n * widths[g])]
+        offs, total = {}, 0
+        for name, sz in sizes:
+            offs[name] = (total, sz)
+            total += (sz + 63) // 64 * 64
+        host = engine._pinned(total)
+        hv = {name: host[o:o + sz] for name, (o, sz) in offs.items()}
+        tok = hv["token_ids"]
+        for i, e in enumerate(entries):
+            tok[cu[i]:cu[i + 1]] = np.asarray(e.tokens, dtype=np.int64)
+            hv["positions"][cu[i]:cu[i + 1]] = np.arange(starts[i], starts[i] + counts[i], dtype=np.int32)
+            hv["seq_of_token"][cu[i]:cu[i + 1]] = i
+        hv["cu_seqlens"][:] = cu
+        hv["seq_slots"][:] = slots
+        hv["seq_starts"][:] = starts
+        hv["logit_rows"][:] = np.asarray(rows, dtype=np.int32)
+        for g in range(n_groups):
+            cache.fill_step(slots, starts, counts, g, hv[f"slot_map{g}"], hv[f"table{g}"].reshape(n, widths[g]))
+        dev = engine._upload(host, total)
+        dv = {name: dev[o:o + sz] for name, (o, sz) in offs.items()}
+        self.tables = [dv[f"table{g}"].view(n, widths[g]) for g in range(n_groups)]
+        self.slot_maps = [dv[f"slot_map{g}"] for g in range(n_groups)]
+        self.ctx = StepContext(
+            T=T, n_seqs=n, token_ids=dv["token_ids"], positions=dv["positions"], seq_of_token=dv["seq_of_token"],
+            cu_seqlens=dv["cu_seqlens"], seq_slots=dv["seq_slots"], seq_starts=dv["seq_starts"],
+            logit_rows=dv["logit_rows"], n_out=n_out,
+            host=HostBatch(slots=slots, starts=starts, counts=counts, cu_seqlens=cu),
+            decode_only=bool(n > 0 and counts.max() == 1), max_count=int(counts.max()) if n else 0)
+        self.host_tokens = tok[:T].copy()
+
+    def layer_cache(self, cache: PagedCache, call: LayerCall) -> LayerCache:
+        state = cache.states.get(call.cache)
+        if call.cache not in cache._group_of:
+            return LayerCache(None, None, None, None, cache.page_size, call.write, state)
+        g = cache.group_of(call.cache)
+        k, v = cache.layer_pages(call.cache)
+        return LayerCache(k, v, self.slot_maps[g], self.tables[g], cache.page_size, call.write, state)
+
+
+class Engine:
+    def __init__(self, model: Union[str, dict, None] = None, *, dtype: str = "bfloat16", page_size: int = 64,
+                 num_pages=None, cache_tokens: Optional[int] = None, max_batch_tokens: int = 2048,
+                 max_requests: int = 8, device: str = "cuda:0", random_weights: bool = False, seed: int = 0,
+                 init_std: float = 0.02, spec: Optional[ModelSpec] = None, tensors: Optional[dict] = None):
+        """``model``: a folder with config.json and model.safetensors; with ``random_weights`` a
+        folder, a config.json path or a config dict whose weights are drawn on the GPU from
+        ``seed``.  ``spec`` (+ ``tensors`` by checkpoint name, or ``random_weights``) builds a
+        model from parts directly, without an architecture."""
+        if dtype not in _DTYPES:
+            raise EngineError(f"dtype {dtype!r} (known: bfloat16, float32)")
+        if not torch.cuda.is_available():
+            raise EngineError("no GPU visible: the engine runs on the GPU only, there is no CPU path")
+        hipops.lib()                      # fail now, loudly, when the kernels cannot be built or loaded
+        self.device = torch.device(device)
+        torch.cuda.set_device(self.device)
+        self.env = Env(_DTYPES[dtype], self.device)
+        self.config = None
+        ckpt_dtype = torch.bfloat16
+        if spec is None:
+            if model is None:
+                raise EngineError("Engine needs a model folder, a configuration or a spec")
+            arch, self.config = read_config(model)
+            spec = arch.build_spec(self.config)
+            ckpt_dtype = _CKPT_DTYPES.get(getattr(self.config, "torch_dtype", "bfloat16"), torch.bfloat16)
+        self.spec = spec
+        self.model = Model(spec, self.env)
+        if tensors is not None:
+            self._load_from_dict(tensors, ckpt_dtype)
+        elif random_weights:
+            self._init_random(seed, init_std)
+        else:
+            if not isinstance(model, str) or not os.path.isdir(model):
+                raise EngineError("without random_weights the model must be a folder with model.safetensors")
+            load_weights(self.model, model, ckpt_dtype)
+        self.page_size, self.max_batch_tokens, self.max_requests = int(page_size), int(max_batch_tokens), int(max_requests)
+        needs = self.model.cache_needs()
+        if num_pages is None:
+            tokens = cache_tokens if cache_tokens is not None else self.max_requests * 4096
+            num_pages = max(1, -(-int(tokens) // self.page_size))
+        self.cache = PagedCache(needs, self.page_size, num_pages, self.max_requests, self.env.dtype, self.device)
+        self._arenas = [Workspace(self.device), Workspace(self.device)]
+        self._step_ws = Workspace(self.device)
+        self._pin = None
+        self._pin_event = None
+        self._meta_dev = None
+        self.steps_run = 0
+
+    # ------------------------------------------------------------------ weights
+    def _load_from_dict(self, tensors: Dict[str, torch.Tensor], ckpt_dtype):
+        from ..weights.loader import resident_dtype, WeightsError
+        plan = self.model.tensor_plan()
+        names = {f for f, _, _, _ in plan}
+        missing = sorted(n for n in names if n not in tensors)
+        unexpected = sorted(n for n in tensors if n not in names)
+        shapes = [(f, tuple(tensors[f].shape), ps.shape) for f, ps, _, _ in plan
+                  if f in tensors and tuple(tensors[f].shape) != tuple(ps.shape)]
+        if missing or unexpected or shapes:
+            raise WeightsError(missing, unexpected, shapes, (), "the given tensors")
+        by_owner = {}
+        for f, ps, owner, local in plan:
+            t = tensors[f]
+            by_owner.setdefault(id(owner), (owner, {}))[1][local] = t.to(
+                device=self.device, dtype=resident_dtype(t.dtype, ps.kind, self.env.dtype, ckpt_dtype))
+        for owner, ts in by_owner.values():
+            owner.load(ts)
+        self.model.finish_loading()
+
+    def _init_random(self, seed: int, std: float):
+        """Draws every tensor on the GPU in its resident dtype: N(0,std), norm weights 1+N(0,std)."""
+        gen = torch.Generator(device=self.device)
+        gen.manual_seed(int(seed))
+        by_owner = {}
+        for f, ps, owner, local in self.model.tensor_plan():
+            if ps.kind == "int":
+                t = torch.zeros(ps.shape, dtype=torch.int32, device=self.device)
+            else:
+                dt = torch.float32 if ps.kind == "vector" else self.env.dtype
+                t = torch.empty(ps.shape, dtype=dt, device=self.device)
+                if ps.init == "zeros":
+                    t.zero_()
+                else:
+                    t.normal_(0.0, std, generator=gen)
+                    if ps.init == "ones":
+                        t += 1.0
+            by_owner.setdefault(id(owner), (owner, {}))[1][local] = t
+        for owner, ts in by_owner.values():
+            owner.load(ts)
+            ts.clear()
+        self.model.finish_loading()
+
+    # ------------------------------------------------------------------ metadata transport
+    def _pinned(self, n: int) -> np.ndarray:
+        if self._pin_event is not None:
+            self._pin_event.synchronize()
+        if self._pin is None or self._pin.numel() < n:
+            self._pin = torch.empty(max(n, 1 << 14), dtype=torch.int32, pin_memory=True)
+            self._pin_np = self._pin.numpy()
+        return self._pin_np
+
+    def _upload(self, host: np.ndarray, n: int) -> torch.Tensor:
+        if self._meta_dev is None or self._meta_dev.numel() < n:
+            self._meta_dev = torch.empty(max(n, 1 << 14), dtype=torch.int32, device=self.device)
+        self._meta_dev[:n].copy_(self._pin[:n], non_blocking=True)
+        self._pin_event = torch.cuda.Event()
+        self._pin_event.record()
+        return self._meta_dev
+
+    # ------------------------------------------------------------------ requests
+    def admit(self) -> int:
+        """A slot for a new request (its state is zeroed)."""
+        return self.cache.admit()
+
+    def release(self, slot: int) -> None:
+        """The request is over: its pages and its slot are given back."""
+        self.cache.release(slot)
+
+    # ------------------------------------------------------------------ the step
+    def step(self, entries: Sequence[StepEntry], commit: bool = True) -> torch.Tensor:
+        """Runs one batch; returns fp32 logits ``[wanted, vocab]`` on the GPU, in the order of
+        the entries and of their ``want``.  Pages for the new positions are reserved here if
+        the caller has not done so; with ``commit`` the positions count as cached afterwards
+        and pages that no later query can read are given back."""
+        if not entries:
+            return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
+        seen = set()
+        V = self.spec.vocab_size
+        total = 0
+        for i, e in enumerate(entries):
+            if e.slot in seen:
+                raise EngineError(f"request slot {e.slot} appears twice in one step")
+            seen.add(e.slot)
+            if not self.cache.live(e.slot):
+                raise EngineError(f"entry {i}: slot {e.slot} holds no request")
+            if len(e.tokens) < 1:
+                raise EngineError(f"entry {i}: no tokens")
+            toks = np.asarray(e.tokens)
+            if toks.min() < 0 or toks.max() >= V:
+                bad = int(toks[(toks < 0) | (toks >= V)][0])
+                raise EngineError(f"entry {i}: token id {bad} outside the vocabulary of {V}")
+            if self.cache.cached(e.slot) + len(e.tokens) > self.spec.max_position:
+                raise EngineError(f"entry {i}: position beyond the model's limit {self.spec.max_position}")
+            total += len(e.tokens)
+        for e in entries:
+            self.cache.reserve(e.slot, len(e.tokens))
+        meta = StepMeta(self, entries)
+        self._step_ws.reset()
+        logits = self.model.forward(meta.ctx, self.cache, meta, self._arenas, self._step_ws)
+        if commit:
+            for e in entries:
+                self.cache.commit(e.slot, len(e.tokens))
+        self.steps_run += 1
+        return logits
+
+    def commit(self, entries: Sequence[StepEntry]) -> None:
+        for e in entries:
+            self.cache.commit(e.slot, len(e.tokens))
+
+    # ------------------------------------------------------------------ convenience
+    def generate(self, prompts, max_tokens: int = 16, temperature: float = 0.0, seed: int = 0, **kw):
+        from .generate import generate
+        return generate(self, prompts, max_tokens=max_tokens, temperature=temperature, seed=seed, **kw)

@@ -1,0 +1,96 @@
+"""A model: blocks built from a ``ModelSpec``, the order in which they run, embedding and
+output matrix.  The same class serves every architecture; what differs is the spec."""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from ..csrc import hipops
+from ..parts import base as P
+from ..parts.base import ParamSpec, PartSpec, CacheNeed
+from ..parts.linear import linear
+from .context import Env, Workspace, StepContext, LayerCache
+
+
+class Model:
+    def __init__(self, spec: P.ModelSpec, env: Env):
+        self.spec, self.env = spec, env
+        self.blocks = [P.build("block", PartSpec(bs.kind, {"spec": bs}), env) for bs in spec.blocks]
+        self.final_norm = P.build("norm", spec.final_norm, env)
+        self.embed: Optional[torch.Tensor] = None
+        self.head: Optional[torch.Tensor] = None
+        for i, call in enumerate(spec.order):
+            if not 0 <= call.block < len(self.blocks):
+                raise ValueError(f"layer call {i} names block {call.block} of {len(self.blocks)}")
+        writers = {}
+        for i, call in enumerate(spec.order):
+            if call.write:
+                if call.cache in writers:
+                    raise ValueError(f"cache {call.cache} is written by layer calls {writers[call.cache]} and {i}")
+                writers[call.cache] = i
+        for i, call in enumerate(spec.order):
+            if not call.write and (call.cache not in writers or writers[call.cache] > i):
+                raise ValueError(f"layer call {i} reads cache {call.cache} before any call has written it")
+        self._writers = writers
+
+    # ------------------------------------------------------------------ tensors
+    def tensor_plan(self) -> List[Tuple[str, ParamSpec, object, str]]:
+        """(checkpoint name, spec, owning part, local name) of every tensor of the model."""
+        plan = []
+        V, d = self.spec.vocab_size, self.spec.hidden_size
+        plan.append((self.spec.embed_name, ParamSpec((V, d)), self, "embed"))
+        if self.spec.head_name is not None:
+            plan.append((self.spec.head_name, ParamSpec((V, d)), self, "head"))
+        for local, ps in self.final_norm.params().items():
+            plan.append((self.spec.final_norm.names[local], ps, self.final_norm, local))
+        for block in self.blocks:
+            for _, part, pspec in block.children:
+                for local, ps in part.params().items():
+                    if local not in pspec.names:
+                        raise KeyError(f"part {pspec.kind!r} declares tensor {local!r} but its spec names no "
+                                       f"checkpoint tensor for it")
+                    plan.append((pspec.names[local], ps, part, local))
+        return plan
+
+    def load(self, tensors: Dict[str, torch.Tensor]):   # the model's own two tensors
+        if "embed" in tensors:
+            self.embed = tensors["embed"].contiguous()
+        if "head" in tensors:
+            self.head = tensors["head"].contiguous()
+
+    def finish_loading(self):
+        if self.embed is None:
+            raise RuntimeError("model has no embedding table")
+        if self.spec.head_name is None:
+            self.head = self.embed
+
+    def cache_needs(self) -> List[Optional[CacheNeed]]:
+        n = max((c.cache for c in self.spec.order), default=-1) + 1
+        needs: List[Optional[CacheNeed]] = [None] * n
+        for cid, i in self._writers.items():
+            needs[cid] = self.blocks[self.spec.order[i].block].mixer.cache_need()
+        return needs
+
+    # ------------------------------------------------------------------ one step
+    def forward(self, ctx: StepContext, cache, meta, arenas, step_ws: Workspace) -> torch.Tensor:
+        """Runs the tokens of the step through every layer call; returns fp32 logits
+        ``[n_out, V]`` at ``ctx.logit_rows``."""
+        T, d = ctx.T, self.spec.hidden_size
+        h = step_ws.take((T, d), torch.float32)
+        hipops.embed(ctx.token_ids, self.embed, h)
+        pending = ()
+        for i, call in enumerate(self.spec.order):
+            ctx.ws = arenas[i % 2]
+            ctx.ws.reset()
+            pending = self.blocks[call.block].forward(h, pending, ctx, meta.layer_cache(cache, call))
+        ctx.ws = arenas[len(self.spec.order) % 2]
+        ctx.ws.reset()
+        if ctx.n_out == 0:
+            return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.env.device)
+        n = ctx.ws.take((ctx.n_out, d), self.env.dtype)
+        self.final_norm.forward(h, n, d1=pending[0] if len(pending) > 0 else None,
+                                d2=pending[1] if len(pending) > 1 else None, rows=ctx.logit_rows, write_h=False)
+        logits = step_ws.take((ctx.n_out, self.spec.vocab_size), torch.float32)
+        linear(n, self.head, logits)
+        return logits

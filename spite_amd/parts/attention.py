@@ -1,0 +1,82 @@
+"""Grouped-query attention over the paged cache.
+
+In order (crates/spite-models/src/llama/llama4.rs:130-207): fused q/k/v projection; position
+encoding of q and k; the weightless RMS norm of every q and k head after the rotation
+(:161-175) if ``qk_norm``; on layers with ``temperature`` the queries times
+ln(floor((pos+1)/floor_scale)+1)*attn_scale+1 (:178-183); keys and values into the cache;
+softmax(q.k/sqrt(hd)) over the keys that the layer's visibility allows
+(crates/spite-compute/src/flash_attn.rs:71-158), head h on kv head h // (H/G); output
+projection.  Scores, softmax and the output sum are fp32.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from .base import Mixer, ParamSpec, CacheNeed, KVNeed, register, build as build_part
+from .linear import linear
+from ..csrc import hipops
+
+
+@register("mixer", "attention")
+class Attention(Mixer):
+    def __init__(self, env, hidden_size, n_heads, n_kv_heads, head_dim, position, visibility="full", span=0,
+                 qk_norm=False, qk_norm_eps=1e-5, temperature=None, softmax_scale=None):
+        if n_heads % n_kv_heads:
+            raise ValueError(f"attention: {n_heads} heads over {n_kv_heads} kv heads")
+        if visibility not in ("full", "chunk", "window"):
+            raise ValueError(f"attention: visibility {visibility!r}")
+        if visibility != "full" and span < 1:
+            raise ValueError(f"attention: {visibility} of size {span}")
+        self.env = env
+        self.d, self.H, self.G, self.hd = int(hidden_size), int(n_heads), int(n_kv_heads), int(head_dim)
+        self.visibility, self.span = visibility, int(span or 0)
+        self.qk_norm, self.qk_norm_eps = bool(qk_norm), float(qk_norm_eps)
+        self.temperature = temperature            # None or (floor_scale, attn_scale)
+        self.scale = float(softmax_scale) if softmax_scale is not None else 1.0 / math.sqrt(self.hd)
+        self.position = build_part("position", position, env)
+        self.wqkv = self.wo = None
+
+    def params(self):
+        d, H, G, hd = self.d, self.H, self.G, self.hd
+        p = {"q_proj": ParamSpec((H * hd, d)), "k_proj": ParamSpec((G * hd, d)),
+             "v_proj": ParamSpec((G * hd, d)), "o_proj": ParamSpec((d, H * hd))}
+        p.update({f"position.{k}": v for k, v in self.position.params().items()})
+        return p
+
+    def load(self, t):
+        # one [(H+2G)*hd, d] operand: the reference splits a fused tensor the same way
+        # (crates/spite-models/src/llama/llama4.rs:130-139)
+        dts = {t[k].dtype for k in ("q_proj", "k_proj", "v_proj")}
+        dt = torch.float32 if len(dts) > 1 else dts.pop()
+        self.wqkv = torch.cat([t["q_proj"].to(dt), t["k_proj"].to(dt), t["v_proj"].to(dt)], dim=0).contiguous()
+        self.wo = t["o_proj"].contiguous()
+        self.position.load({k[len("position."):]: v for k, v in t.items() if k.startswith("position.")})
+
+    def cache_need(self):
+        return CacheNeed(kv=KVNeed(self.G, self.hd, self.visibility, self.span))
+
+    def forward(self, x, ctx, cache):
+        T = x.shape[0]
+        H, G, hd = self.H, self.G, self.hd
+        ws = ctx.ws
+        qkv = ws.take((T, (H + 2 * G) * hd), x.dtype)
+        linear(x, self.wqkv, qkv)
+        pe = self.position
+        if not pe.fused:
+            pe.transform(qkv, ctx.positions, H, G, hd)
+        ka = pe.kernel_args() if pe.fused else {"use_rope": False, "inv_freq": None, "adjacent": False}
+        q = ws.take((T, H * hd), x.dtype)
+        temp = self.temperature
+        hipops.rope_kvwrite(qkv, q, cache.k_pages, cache.v_pages, ctx.positions, cache.slot_map, ka["inv_freq"],
+                            H, G, hd, cache.page_size, use_rope=ka["use_rope"], adjacent=ka["adjacent"],
+                            use_norm=self.qk_norm, norm_eps=self.qk_norm_eps, use_temp=temp is not None,
+                            floor_scale=temp[0] if temp else 1, attn_scale=temp[1] if temp else 0.0,
+                            write_kv=cache.write)
+        o = ws.take((T, H * hd), x.dtype)
+        hipops.attn_generic(q, cache.k_pages, cache.v_pages, o, ctx.positions, ctx.seq_of_token,
+                            cache.block_table, T, H, G, hd, cache.page_size, self.visibility, self.span, self.scale)
+        out = ws.take((T, self.d), torch.float32)
+        linear(o, self.wo, out)
+        return out

@@ -1,0 +1,172 @@
+"""Interfaces of the parts that a layer is put together from, and their registries.
+
+A model is described by data: a ``ModelSpec`` holds one ``BlockSpec`` per layer (which norm,
+which mixer, which feed-forward, each with its own sizes and constants and the names of its
+tensors in the checkpoint) and an ``order``: the list of layer calls of one step.  A call
+names the block to run and the cache it works on, so a block may run twice and a layer may
+read the cache that another layer wrote.  No part knows which model it is in.
+
+Every kind of part is a class registered under a name; a ``PartSpec`` names the kind and
+carries the constructor's keyword arguments.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, List, Optional, Tuple
+
+import torch
+
+
+@dataclass(frozen=True)
+class ParamSpec:
+    """One tensor of a part, in the layout of the checkpoint."""
+    shape: Tuple[int, ...]
+    kind: str = "matrix"    # "matrix": computed in the run's dtype; "vector": always fp32; "int": int32
+    init: str = "normal"    # random-weights mode: "normal" N(0,std), "ones" 1+N(0,std), "zeros"
+
+
+@dataclass(frozen=True)
+class KVNeed:
+    """Keys and values in pages: heads, head size and which keys a query may read."""
+    n_kv_heads: int
+    head_dim: int
+    visibility: str = "full"          # "full" | "chunk" | "window"
+    span: int = 0                     # chunk size or window
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """Per-request state of fixed size: a tensor of this shape for every request slot."""
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass(frozen=True)
+class CacheNeed:
+    kv: Optional[KVNeed] = None
+    state: Optional[StateNeed] = None
+
+
+@dataclass
+class PartSpec:
+    kind: str
+    args: Dict[str, Any] = field(default_factory=dict)
+    names: Dict[str, str] = field(default_factory=dict)   # local tensor name -> checkpoint name
+
+
+@dataclass
+class BlockSpec:
+    kind: str                    # arrangement, e.g. "prenorm"
+    norm1: PartSpec
+    mixer: PartSpec
+    norm2: PartSpec
+    ffn: PartSpec
+
+
+@dataclass(frozen=True)
+class LayerCall:
+    block: int                   # index into ModelSpec.blocks
+    cache: int                   # cache id; the call with write=True fills it
+    write: bool = True
+
+
+@dataclass
+class ModelSpec:
+    architecture: str
+    vocab_size: int
+    hidden_size: int
+    blocks: List[BlockSpec]
+    order: List[LayerCall]
+    final_norm: PartSpec
+    embed_name: str
+    head_name: Optional[str]     # None: the embedding table is the output matrix
+    eos_token_ids: Tuple[int, ...] = ()
+    max_position: int = 1 << 20
+
+
+class Part:
+    """Base of all parts: declares its tensors and takes them when they are loaded."""
+
+    def params(self) -> Dict[str, ParamSpec]:
+        return {}
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        """``tensors``: local name -> tensor on the GPU, already in its resident dtype."""
+
+
+class Norm(Part):
+    def forward(self, h, out, *, d1=None, d2=None, out32=None, rows=None, write_h=True) -> None:
+        """h (fp32 [T,d]) += d1 + d2 (kept if write_h); out[i] (and out32[i]) = norm(h[r]), r =
+        rows[i] or i."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    #: True when the fused rotation kernel applies this encoding (see kernel_args).
+    fused = True
+
+    def kernel_args(self) -> Dict[str, Any]:
+        return {"use_rope": False, "inv_freq": None, "adjacent": False}
+
+    def transform(self, qkv, positions, n_heads, n_kv_heads, head_dim) -> None:
+        """For encodings the fused kernel does not know: change q and k of the fused
+        projection's rows in place before they are normed and cached."""
+
+
+class Mixer(Part):
+    def cache_need(self) -> CacheNeed:
+        return CacheNeed()
+
+    def forward(self, x, ctx, cache):
+        """x [T,d] in the run's dtype -> fp32 [T,d], the residual's increment, taken from
+        ``ctx.ws`` (it must stay valid until the next layer call has consumed it)."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    #: ask the block for the normed input in fp32 as well (routers want it)
+    wants_f32_input = False
+
+    def forward(self, x, x32, ctx):
+        """x [T,d] (x32: the same in fp32, if asked for) -> a tuple of one or two fp32 [T,d]
+        increments of the residual, taken from ``ctx.ws``."""
+        raise NotImplementedError
+
+
+class Block(Part):
+    def forward(self, h, pending, ctx, cache):
+        """Runs the layer on the residual stream h (fp32 [T,d]); ``pending`` are up to two
+        increments not yet added to h.  Returns the new pending increments."""
+        raise NotImplementedError
+
+
+# ----------------------------------------------------------------------------- registries
+_REGISTRIES: Dict[str, Dict[str, Callable]] = {
+    "norm": {}, "position": {}, "mixer": {}, "ffn": {}, "block": {},
+}
+
+
+class UnknownPart(KeyError):
+    pass
+
+
+def register(category: str, kind: str, cls=None):
+    """``register("mixer", "attention", Attention)`` or as a decorator."""
+    if category not in _REGISTRIES:
+        raise KeyError(f"no part category {category!r} (known: {sorted(_REGISTRIES)})")
+
+    def deco(c):
+        _REGISTRIES[category][kind] = c
+        return c
+    return deco(cls) if cls is not None else deco
+
+
+def build(category: str, spec: PartSpec, env) -> Part:
+    reg = _REGISTRIES[category]
+    if spec.kind not in reg:
+        raise UnknownPart(f"no {category} of kind {spec.kind!r} is registered (known: {sorted(reg)})")
+    return reg[spec.kind](env=env, **spec.args)
+
+
+def registered(category: str):
+    return sorted(_REGISTRIES[category])

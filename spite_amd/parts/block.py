@@ -1,0 +1,36 @@
+"""Arrangement of a layer: pre-norm residual block,
+h += mixer(norm1(h)); h += ffn(norm2(h)) (crates/spite-models/src/llama/llama4.rs:126-127,
+202-211, 272-274).  The additions are folded into the norm that follows them: a block hands
+its last increments to the next block (or the final norm) instead of adding them itself."""
+from __future__ import annotations
+
+import torch
+
+from .base import Block, register, build as build_part
+
+
+@register("block", "prenorm")
+class PreNormBlock(Block):
+    def __init__(self, env, spec):
+        self.env = env
+        self.norm1 = build_part("norm", spec.norm1, env)
+        self.mixer = build_part("mixer", spec.mixer, env)
+        self.norm2 = build_part("norm", spec.norm2, env)
+        self.ffn = build_part("ffn", spec.ffn, env)
+        self.children = (("norm1", self.norm1, spec.norm1), ("mixer", self.mixer, spec.mixer),
+                         ("norm2", self.norm2, spec.norm2), ("ffn", self.ffn, spec.ffn))
+
+    def forward(self, h, pending, ctx, cache):
+        T, d = h.shape
+        ws = ctx.ws
+        d1 = pending[0] if len(pending) > 0 else None
+        d2 = pending[1] if len(pending) > 1 else None
+        n = ws.take((T, d), self.env.dtype)
+        self.norm1.forward(h, n, d1=d1, d2=d2)
+        delta = self.mixer.forward(n, ctx, cache)
+        n2 = ws.take((T, d), self.env.dtype)
+        n2_32 = None
+        if self.ffn.wants_f32_input:
+            n2_32 = n2 if n2.dtype == torch.float32 else ws.take((T, d), torch.float32)
+        self.norm2.forward(h, n2, d1=delta, out32=None if n2_32 is n2 else n2_32)
+        return tuple(self.ffn.forward(n2, n2_32, ctx))

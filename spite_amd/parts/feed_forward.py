@@ -1,0 +1,102 @@
+"""Feed-forward parts.
+
+``dense_glu`` (crates/spite-models/src/llama/llama4.rs:257-271):
+y = W_down . (silu(W_gate . x) * (W_up . x)).
+
+``moe_top1_sigmoid`` (crates/spite-models/src/moe.rs:87-194, llama4.rs:212-256): router
+logits W_r . x in fp32; the expert with the largest logit (lowest index on ties); its
+*input* is x * sigmoid(logit), its output is not weighted; a shared expert on the unscaled
+x is added.  Routed and shared experts run as one grouped product over a row list: group
+e < E holds the tokens routed to expert e, group E every token.
+"""
+from __future__ import annotations
+
+import torch
+
+from .base import FeedForward, ParamSpec, register
+from .linear import linear
+from ..csrc import hipops
+
+
+@register("ffn", "dense_glu")
+class DenseGLU(FeedForward):
+    def __init__(self, env, hidden_size, intermediate_size):
+        self.d, self.F = int(hidden_size), int(intermediate_size)
+        self.w_gate_up = self.w_down = None
+
+    def params(self):
+        return {"gate_proj": ParamSpec((self.F, self.d)), "up_proj": ParamSpec((self.F, self.d)),
+                "down_proj": ParamSpec((self.d, self.F))}
+
+    def load(self, t):
+        dt = t["gate_proj"].dtype if t["gate_proj"].dtype == t["up_proj"].dtype else torch.float32
+        self.w_gate_up = torch.cat([t["gate_proj"].to(dt), t["up_proj"].to(dt)], dim=0).contiguous()
+        self.w_down = t["down_proj"].contiguous()
+
+    def forward(self, x, x32, ctx):
+        T = x.shape[0]
+        act = ctx.ws.take((T, self.F), x.dtype)
+        linear(x, self.w_gate_up, act, glu=True)
+        y = ctx.ws.take((T, self.d), torch.float32)
+        linear(act, self.w_down, y)
+        return (y,)
+
+
+@register("ffn", "moe_top1_sigmoid")
+class MoeTop1Sigmoid(FeedForward):
+    wants_f32_input = True
+
+    def __init__(self, env, hidden_size, intermediate_size, n_experts, shared_intermediate_size=None):
+        self.d, self.F, self.E = int(hidden_size), int(intermediate_size), int(n_experts)
+        self.Fs = int(shared_intermediate_size if shared_intermediate_size is not None else intermediate_size)
+        if self.E < 1 or self.E > 65000:
+            raise ValueError(f"moe: {self.E} experts")
+        self.fused_shared = self.Fs == self.F
+        self.w_router = self.w_gate_up = self.w_down = None
+        self.ws_gate_up = self.ws_down = None
+
+    def params(self):
+        d, F, Fs, E = self.d, self.F, self.Fs, self.E
+        return {"router": ParamSpec((E, d), kind="vector"),
+                "experts.gate_up_proj": ParamSpec((E, d, 2 * F)), "experts.down_proj": ParamSpec((E, F, d)),
+                "shared.gate_proj": ParamSpec((Fs, d)), "shared.up_proj": ParamSpec((Fs, d)),
+                "shared.down_proj": ParamSpec((d, Fs))}
+
+    def load(self, t):
+        self.w_router = t["router"].contiguous()
+        # checkpoint [E, d, 2F] (x @ M) -> [E, 2F, d] rows of gate then up; down [E, F, d] -> [E, d, F]
+        gu = t["experts.gate_up_proj"].transpose(1, 2)
+        dn = t["experts.down_proj"].transpose(1, 2)
+        sgu = torch.cat([t["shared.gate_proj"], t["shared.up_proj"]], dim=0)
+        sdn = t["shared.down_proj"]
+        if self.fused_shared and sgu.dtype == gu.dtype and sdn.dtype == dn.dtype:
+            self.w_gate_up = torch.cat([gu, sgu[None]], dim=0).contiguous()
+            self.w_down = torch.cat([dn, sdn[None]], dim=0).contiguous()
+        else:
+            self.fused_shared = False
+            self.w_gate_up, self.w_down = gu.contiguous(), dn.contiguous()
+            self.ws_gate_up, self.ws_down = sgu.contiguous(), sdn.contiguous()
+
+    def forward(self, x, x32, ctx):
+        T, E, F, d = x.shape[0], self.E, self.F, self.d
+        ws = ctx.ws
+        expert = ws.take((T,), torch.int32)
+        weight = ws.take((T,), torch.float32)
+        hipops.router_top1(x32, self.w_router, expert, weight)
+        n = 2 * T if self.fused_shared else T
+        src, dst = ws.take((n,), torch.int32), ws.take((n,), torch.int32)
+        scale = ws.take((n,), torch.float32)
+        groups = E + 1 if self.fused_shared else E
+        offsets = ws.take((groups + 1,), torch.int32)
+        hipops.moe_plan(expert, weight, src, scale, dst, offsets, T, E, self.fused_shared)
+        act = ws.take((n, F), x.dtype)
+        linear(x, self.w_gate_up, act, glu=True, offsets=offsets, n_groups=groups, a_rows=src, a_scale=scale, rows=n)
+        # slot s writes row dst[s]: rows [0,T) the routed result per token, rows [T,2T) the shared one
+        y = ws.take((2 * T, d), torch.float32)
+        linear(act, self.w_down, y, offsets=offsets, n_groups=groups, y_rows=dst, rows=n)
+        if self.fused_shared:
+            return (y[:T], y[T:])
+        act_s = ws.take((T, self.Fs), x.dtype)
+        linear(x, self.ws_gate_up, act_s, glu=True)
+        linear(act_s, self.ws_down, y[T:])
+        return (y[:T], y[T:])

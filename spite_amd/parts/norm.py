@@ -1,0 +1,24 @@
+"""RMSNorm (crates/spite-models/src/dense.rs:175-181): y = x * 1/sqrt(mean(x^2) + eps) * w,
+sum and scale in fp32, fused with the residual additions that precede it."""
+from __future__ import annotations
+
+from .base import Norm, ParamSpec, register
+from ..csrc import hipops
+
+
+@register("norm", "rms")
+class RMSNorm(Norm):
+    def __init__(self, env, width: int, eps: float):
+        self.width = int(width)
+        self.eps = float(eps)
+        self.weight = None
+
+    def params(self):
+        return {"weight": ParamSpec((self.width,), kind="vector", init="ones")}
+
+    def load(self, tensors):
+        self.weight = tensors["weight"]
+
+    def forward(self, h, out, *, d1=None, d2=None, out32=None, rows=None, write_h=True):
+        hipops.add_rmsnorm(h, self.weight, self.eps, out=out, out32=out32, d1=d1, d2=d2, rows=rows,
+                           n_rows=(rows.numel() if rows is not None else h.shape[0]), write_h=write_h)

@@ -1,0 +1,101 @@
+"""Sampling on the GPU, in the order of the reference's pipeline
+(crates/spite-sampling/src/lib.rs:273-296): repetition penalty (window ``repeat_last_n``, each
+distinct id once) -> /temperature -> min-p -> top-k -> top-p -> greedy when temperature <= 0,
+else the inverse-CDF draw with one LCG stream per request (:343-348).  Names and meanings of
+the options are the reference's ``SamplerConfig`` (:83-111); the defaults here switch every
+filter off.  Greedy takes the lowest index among equal maxima.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import List, Sequence
+
+import numpy as np
+import torch
+
+from ..csrc import hipops
+
+LCG_MUL = 6364136223846793005
+LCG_ADD = 1442695040888963407
+_MASK = (1 << 64) - 1
+
+
+def lcg_next(state: int):
+    """crates/spite-sampling/src/lib.rs:343-348: returns (new state, u in [0,1) as float32)."""
+    state = (state * LCG_MUL + LCG_ADD) & _MASK
+    return state, float(np.float32(state >> 33) / np.float32(2147483648.0))
+
+
+@dataclass
+class SamplingParams:
+    temperature: float = 0.0          # <= 0: greedy
+    top_k: int = 0                    # 0 = off
+    top_p: float = 1.0                # 1.0 = off
+    min_p: float = 0.0                # 0 = off
+    repetition_penalty: float = 1.0   # 1.0 = off
+    repeat_last_n: int = 64           # 0 = the whole context
+    seed: int = 0
+
+    def filters(self) -> bool:
+        return (self.top_k > 0 or self.top_p < 1.0 or self.min_p > 0.0
+                or abs(self.repetition_penalty - 1.0) >= 1.1920929e-07)
+
+
+class Sampler:
+    def __init__(self, device):
+        self.device = device
+
+    def _process_row(self, row: torch.Tensor, p: SamplingParams, context: Sequence[int]) -> torch.Tensor:
+        l = row.clone()
+        V = l.numel()
+        if abs(p.repetition_penalty - 1.0) >= 1.1920929e-07 and len(context):
+            win = context if p.repeat_last_n == 0 or p.repeat_last_n >= len(context) else context[-p.repeat_last_n:]
+            ids = sorted({int(t) for t in win if 0 <= int(t) < V})
+            if ids:
+                idx = torch.tensor(ids, dtype=torch.long, device=l.device)
+                v = l[idx]
+                l[idx] = torch.where(v > 0, v / p.repetition_penalty, v * p.repetition_penalty)
+        if p.temperature > 0:
+            l = l / p.temperature
+        if p.min_p > 0:
+            l = l.masked_fill(l < l.max() + math.log(p.min_p), float("-inf"))
+        if 0 < p.top_k < V:
+            thresh = torch.topk(l, p.top_k).values[-1]
+            l = l.masked_fill(l < thresh, float("-inf"))
+        if p.top_p < 1.0:
+            vals, order = torch.sort(l, descending=True, stable=True)
+            e = torch.exp(vals - vals[0])
+            total = e.sum()
+            cum = torch.cumsum(e, 0) / total
+            reached = (cum >= p.top_p).nonzero()
+            kept = int(reached[0]) + 1 if reached.numel() else V
+            l[order[max(kept, 1):]] = float("-inf")
+        return l
+
+    def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], contexts: Sequence[Sequence[int]],
+               rng_states: List[int]) -> List[int]:
+        """One token per row of ``logits`` (fp32 ``[n, V]``).  ``rng_states[i]`` is advanced for
+        every row that draws."""
+        n = logits.shape[0]
+        if n == 0:
+            return []
+        temps = np.zeros(n, dtype=np.float32)
+        us = np.zeros(n, dtype=np.float32)
+        work = logits
+        if any(p.filters() for p in params):
+            work = logits.clone()
+            for i, p in enumerate(params):
+                if p.filters():
+                    work[i] = self._process_row(logits[i], p, contexts[i])
+        for i, p in enumerate(params):
+            if p.temperature > 0:
+                temps[i] = 1.0 if p.filters() else p.temperature     # filtered rows are divided already
+                rng_states[i], us[i] = lcg_next(rng_states[i])
+        out = torch.empty(n, dtype=torch.int32, device=logits.device)
+        if temps.max() <= 0:
+            hipops.sample_rows(work, None, None, out, n)
+        else:
+            both = torch.from_numpy(np.stack([temps, us])).to(logits.device)
+            hipops.sample_rows(work, both[0], both[1], out, n)
+        return [int(x) for x in out.cpu().tolist()]
