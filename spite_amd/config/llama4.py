@@ -166,7 +166,8 @@ class Llama4Config:
             max_position_embeddings=opt("max_position_embeddings", int, 1 << 20),
             torch_dtype=opt("torch_dtype", str, "bfloat16"),
             bos_token_id=src.get("bos_token_id"), eos_token_ids=eos)
-        problems += cfg._inconsistencies()
+        missing = {m.split("'")[1] for m in problems if m.startswith("missing key")}
+        problems += [m for m in cfg._inconsistencies() if m.split(" ")[0] not in missing]
         if problems:
             raise ConfigError("config.json: " + "; ".join(problems))
         return cfg
@@ -187,9 +188,7 @@ class Llama4Config:
         for key, val in pos.items():
             if val < 1:
                 p.append(f"{key} must be >= 1, got {val}")
-        if p:
-            return p
-        if self.num_attention_heads % self.num_key_value_heads:
+        if self.num_key_value_heads >= 1 and self.num_attention_heads % self.num_key_value_heads:
             p.append(f"num_attention_heads {self.num_attention_heads} is not a multiple of "
                      f"num_key_value_heads {self.num_key_value_heads}")
         if self.head_dim % 2:

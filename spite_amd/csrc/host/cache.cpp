@@ -121,16 +121,16 @@ int CacheManager::release(int slot) {
 int64_t CacheManager::peak_pages(int64_t total, int64_t portion, int g) const {
     const int64_t ps = page_size_;
     if (groups_[g].kind == VIS_FULL || portion < 1) return (total + ps - 1) / ps;
-    // Walk the portions: before a portion the request holds blocks [frontier/ps, ceil(c/ps)),
-    // during it up to ceil((c+n)/ps).
-    int64_t peak = 0;
-    for (int64_t c = 0; c < total; c += portion) {
-        const int64_t n = std::min(portion, total - c);
-        const int64_t low = first_visible(c, groups_[g].kind, groups_[g].span) / ps;
-        const int64_t high = (c + n + ps - 1) / ps;
-        peak = std::max(peak, high - low);
-    }
-    return peak;
+    // A portion of n positions that starts at c reads from first_visible(c), at most span-1
+    // positions before c.  Portions start anywhere (the budget cuts them), so take the worst
+    // alignment; chunks that are whole pages start on a page.
+    const int64_t all = (total + ps - 1) / ps;
+    const int64_t n = std::min(portion, total);
+    const int64_t span = groups_[g].span;
+    int64_t worst;
+    if (groups_[g].kind == VIS_CHUNK && span % ps == 0) worst = (span - 1 + n + ps - 1) / ps;
+    else worst = (span + n - 2) / ps + 2;
+    return std::min(all, worst);
 }
 
 void CacheManager::slot_mapping(int slot, int g, int64_t start, int64_t n, int32_t* out) const {

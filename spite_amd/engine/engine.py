@@ -225,11 +225,13 @@ class Engine:
         self.cache.release(slot)
 
     # ------------------------------------------------------------------ the step
-    def step(self, entries: Sequence[StepEntry], commit: bool = True) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], commit: bool = True, trace: Optional[dict] = None) -> torch.Tensor:
         """Runs one batch; returns fp32 logits ``[wanted, vocab]`` on the GPU, in the order of
         the entries and of their ``want``.  Pages for the new positions are reserved here if
         the caller has not done so; with ``commit`` the positions count as cached afterwards
-        and pages that no later query can read are given back."""
+        and pages that no later query can read are given back.  ``trace``, a dict, is a
+        testing aid: parts leave what they decided in it (``moe_experts``: one int32 tensor
+        ``[tokens]`` per layer call with experts, in the order of the calls)."""
         if not entries:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
         seen = set()
@@ -253,6 +255,8 @@ class Engine:
         for e in entries:
             self.cache.reserve(e.slot, len(e.tokens))
         meta = StepMeta(self, entries)
+        if trace is not None:
+            meta.ctx.extras["trace"] = trace
         self._step_ws.reset()
         logits = self.model.forward(meta.ctx, self.cache, meta, self._arenas, self._step_ws)
         if commit:

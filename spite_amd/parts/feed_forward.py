@@ -83,6 +83,8 @@ class MoeTop1Sigmoid(FeedForward):
         expert = ws.take((T,), torch.int32)
         weight = ws.take((T,), torch.float32)
         hipops.router_top1(x32, self.w_router, expert, weight)
+        if ctx.extras.get("trace") is not None:      # a testing aid: which expert each row took
+            ctx.extras["trace"].setdefault("moe_experts", []).append(expert.clone())
         n = 2 * T if self.fused_shared else T
         src, dst = ws.take((n,), torch.int32), ws.take((n,), torch.int32)
         scale = ws.take((n,), torch.float32)

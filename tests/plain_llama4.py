@@ -158,9 +158,15 @@ def swiglu_mlp(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down
     return (silu(x @ w_gate.T) * (x @ w_up.T)) @ w_down.T
 
 
-def router_top1(x: torch.Tensor, w_router: torch.Tensor):
+def router_top1(x: torch.Tensor, w_router: torch.Tensor, hints=None, hint_rel: float = 0.0, taken=None):
     """crates/spite-models/src/moe.rs:65-66,110-126: logits = W_r.x; pick by raw logit,
-    descending, stable sort so that ties go to the lowest index; weight = sigmoid(logit)."""
+    descending, stable sort so that ties go to the lowest index; weight = sigmoid(logit).
+
+    ``hints[t]`` (optional) names the expert that another implementation chose for row t.
+    Where it differs from the choice made here and the two logits lie within ``hint_rel``
+    times the largest |logit| of the row, the two experts are tied at that implementation's
+    precision and the hint is followed (and counted in ``taken``); a hint further off is
+    ignored."""
     logits = x @ w_router.T
     E = logits.shape[-1]
     idx = torch.zeros(logits.shape[0], dtype=torch.int64)
@@ -169,13 +175,19 @@ def router_top1(x: torch.Tensor, w_router: torch.Tensor):
         for e in range(1, E):
             if logits[t, e] > logits[t, best]:
                 best = e
+        if hints is not None and int(hints[t]) != best and 0 <= int(hints[t]) < E:
+            gap = float(logits[t, best] - logits[t, int(hints[t])])
+            if gap <= hint_rel * float(logits[t].abs().max()):
+                best = int(hints[t])
+                if taken is not None:
+                    taken.append(t)
         idx[t] = best
     chosen = logits.gather(1, idx[:, None])[:, 0]
     w = 1.0 / (1.0 + torch.exp(-chosen))
     return idx, w, logits
 
 
-def moe_ffn(x, w_router, gate_up, down, sh_gate, sh_up, sh_down) -> torch.Tensor:
+def moe_ffn(x, w_router, gate_up, down, sh_gate, sh_up, sh_down, hints=None, hint_rel=0.0, taken=None, chosen=None) -> torch.Tensor:
     """crates/spite-models/src/moe.rs:168-191 and llama4.rs:231-256.
 
     Routed: the expert's *input* is x*w (moe.rs:172-173), the output is not weighted
@@ -183,7 +195,9 @@ def moe_ffn(x, w_router, gate_up, down, sh_gate, sh_up, sh_down) -> torch.Tensor
     added (llama4.rs:253-255).  ``gate_up`` is ``[E, d, 2F]`` (gate = first F columns),
     ``down`` ``[E, F, d]``: the file layout, applied as x @ M.
     """
-    idx, w, _ = router_top1(x, w_router)
+    idx, w, _ = router_top1(x, w_router, hints, hint_rel, taken)
+    if chosen is not None:
+        chosen.extend(idx.tolist())
     F_ = down.shape[1]
     y = torch.zeros_like(x)
     for t in range(x.shape[0]):
@@ -215,7 +229,8 @@ def layer_kinds(cfg: dict):
 
 
 def forward(cfg: dict, weights: dict, tokens, start_pos: int = 0, dtype=torch.float64,
-            visibility: str = "chunk") -> torch.Tensor:
+            visibility: str = "chunk", route_hints=None, hint_rel: float = 0.0, taken=None,
+            chosen=None) -> torch.Tensor:
     """Logits ``[T, V]`` of one whole sequence (crates/spite-models/src/llama/llama4.rs:74-283,
     layer-major instead of token-major; same arithmetic).  ``visibility`` of the rotating
     layers: ``chunk`` (configuration) or ``window`` (what the reference computes)."""
@@ -257,9 +272,14 @@ def forward(cfg: dict, weights: dict, tokens, start_pos: int = 0, dtype=torch.fl
         n = rms_norm(h, W[p + "post_attention_layernorm.weight"], eps)  # :210-211
         f = p + "feed_forward."
         if is_moe[L]:
+            took = []
             y = moe_ffn(n, W[f + "router.weight"], W[f + "experts.gate_up_proj"], W[f + "experts.down_proj"],
                         W[f + "shared_expert.gate_proj.weight"], W[f + "shared_expert.up_proj.weight"],
-                        W[f + "shared_expert.down_proj.weight"])    # :212-256
+                        W[f + "shared_expert.down_proj.weight"],    # :212-256
+                        None if route_hints is None else route_hints.get(L), hint_rel, took,
+                        None if chosen is None else chosen.setdefault(L, []))
+            if taken is not None:
+                taken.extend((L, t) for t in took)
         else:
             y = swiglu_mlp(n, W[f + "gate_proj.weight"], W[f + "up_proj.weight"], W[f + "down_proj.weight"])
         h = h + y                                                   # :272-274
