@@ -3,8 +3,9 @@ the host-side bookkeeping in the native cache manager.
 
 Layers are grouped by what they need: the same number of kv heads, head size and
 visibility (every key, the query's chunk, a window).  A group's pool is one tensor
-``[layers, 2, pages, kv_heads, page_size, head_dim]``; a page is the same row range in every
-layer of the group, so one block table serves all of them.
+``[layers, 2, pages, kv_heads, page_size, head_dim]`` (the value half is used transposed,
+``[pages, kv_heads, head_dim, page_size]``); a page is the same row range in every layer of
+the group, so one block table serves all of them.
 """
 from __future__ import annotations
 
@@ -184,4 +185,6 @@ class PagedCache:
     def layer_pages(self, cache_id: int):
         g = self.groups[self._group_of[cache_id]]
         li = self._layer_in_group[cache_id]
-        return g.kv[li, 0], g.kv[li, 1]
+        G, hd = g.key[0], g.key[1]
+        # keys [pages, G, page_size, hd]; values transposed in the same bytes: [pages, G, hd, page_size]
+        return g.kv[li, 0], g.kv[li, 1].view(g.n_pages, G, hd, self.page_size)

@@ -1,0 +1,205 @@
+// Decode attention over the paged cache on MFMA: one query token per request, the visible
+// keys of a request split over workgroups ("split-KV"), partial (max, sum, output) per split
+// in fp32, then a small kernel that combines the splits.
+//
+// A workgroup serves one token, one kv head and one split; the H/G query heads that share
+// the kv head are the 16 columns of the MFMA tiles (unused columns are zero), so K and V are
+// read once for all of them.  Its four waves take the split's 32-key blocks in turn.
+//   S^T[keys x heads] = K[keys x hd] . Q^T            (A = K rows as they lie in the page)
+//   O^T[hd x heads]  += V^T[hd x keys] . P^T          (A = value page, stored transposed)
+// The softmax runs down the columns: a lane holds eight keys of one head, the other keys of
+// that head sit in the lanes 16, 32 and 48 further on.  P^T is fed to the second product in
+// the order in which the first one left it; V^T is read in the same order of keys.
+// Scores, running maximum and sum, and the output are fp32; P is rounded to bf16 only as an
+// MFMA operand.
+#include "common.h"
+
+template <int HD>
+__global__ __launch_bounds__(256)
+void attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages,
+                        const bf16* __restrict__ v_pages, float* __restrict__ part,
+                        const int* __restrict__ positions, const int* __restrict__ seq_of_token,
+                        const int* __restrict__ block_table, int max_blocks, int H, int G, int ps, int vis,
+                        int span, float scale_log2e, int n_splits) {
+    constexpr int NC = HD / 32;      // 32-wide chunks of the head for the score product
+    constexpr int ND = HD / 16;      // 16-row tiles of the output
+    constexpr int ROW = HD + 2;      // partial record: output, max, sum
+    extern __shared__ float sm[];    // [4 waves][16 heads][ROW]
+    const int split = blockIdx.x, g = blockIdx.y, t = blockIdx.z;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n = lane & 15, qd = lane >> 4;
+    const int QH = H / G;
+    const int p = positions[t];
+    const int lo = sp_first_visible(p, vis, span);
+    const int* bt = block_table + (size_t)seq_of_token[t] * max_blocks;
+
+    const int b_first = lo / 32, b_last = p / 32;
+    const int nblk = b_last - b_first + 1;
+    const int per = (nblk + n_splits - 1) / n_splits;
+    const int rb = b_first + split * per;
+    const int re = (rb + per < b_last + 1) ? rb + per : b_last + 1;
+
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    bf16x8 qf[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+        qf[c] = n < QH ? *(const bf16x8*)(q + ((size_t)t * H + g * QH + n) * HD + c * 32 + qd * 8) : zero8;
+
+    float m_run = -INFINITY, l_run = 0.f;
+    f32x4 o[ND];
+#pragma unroll
+    for (int d = 0; d < ND; ++d) o[d] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    for (int kb = rb + wave; kb < re; kb += 4) {
+        const int key0 = kb * 32;
+        const int page = bt[key0 / ps];
+        const int off0 = key0 % ps;
+        const size_t pg = (size_t)(page < 0 ? 0 : page) * G + g;
+        const bf16* kbase = k_pages + (pg * ps + off0) * HD;
+        const bf16* vbase = v_pages + pg * HD * ps + off0;
+        bf16x8 kf[2][NC];
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int c = 0; c < NC; ++c)
+                kf[tt][c] = *(const bf16x8*)(kbase + (size_t)(tt * 16 + n) * HD + c * 32 + qd * 8);
+        bf16x4 vf[ND][2];
+#pragma unroll
+        for (int d = 0; d < ND; ++d)
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt)
+                vf[d][tt] = *(const bf16x4*)(vbase + (size_t)(d * 16 + n) * ps + tt * 16 + qd * 4);
+
+        f32x4 s[2];
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+            s[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < NC; ++c)
+                s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[tt][c], qf[c], s[tt], 0, 0, 0);
+        }
+        float mx = -INFINITY;
+        bool ok[2][4];
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int j = key0 + tt * 16 + qd * 4 + i;
+                ok[tt][i] = j >= lo && j <= p;
+                const float v = ok[tt][i] ? (page < 0 ? NAN : s[tt][i] * scale_log2e) : -INFINITY;
+                s[tt][i] = v;
+                mx = fmaxf(mx, v);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run, mx);
+        const float alpha = (m_run == -INFINITY) ? 0.f : exp2f(m_run - m_new);
+        float sum = 0.f;
+        bf16x8 pf;
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float e = ok[tt][i] ? exp2f(s[tt][i] - m_new) : 0.f;
+                sum += e;
+                pf[tt * 4 + i] = (bf16)e;
+            }
+        sum += __shfl_xor(sum, 16, 64);
+        sum += __shfl_xor(sum, 32, 64);
+        l_run = l_run * alpha + sum;
+        m_run = m_new;
+#pragma unroll
+        for (int d = 0; d < ND; ++d) {
+            bf16x8 va;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { va[e] = vf[d][0][e]; va[4 + e] = vf[d][1][e]; }
+            o[d] = o[d] * alpha;
+            o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pf, o[d], 0, 0, 0);
+        }
+    }
+
+    // the four waves' partial results meet in LDS; o[d][i] of lane (n, qd) is O[head n][d*16 + qd*4 + i]
+    float* mine = sm + ((size_t)wave * 16 + n) * ROW;
+#pragma unroll
+    for (int d = 0; d < ND; ++d)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mine[d * 16 + qd * 4 + i] = o[d][i];
+    if (qd == 0) { mine[HD] = m_run; mine[HD + 1] = l_run; }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < QH * ROW; idx += 256) {
+        const int hn = idx / ROW, c = idx % ROW;
+        float M = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) M = fmaxf(M, sm[((size_t)w * 16 + hn) * ROW + HD]);
+        float acc = 0.f;
+        if (c == HD) acc = M;
+        else {
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const float mw = sm[((size_t)w * 16 + hn) * ROW + HD];
+                const float f = (mw == -INFINITY) ? 0.f : exp2f(mw - M);
+                acc += f * sm[((size_t)w * 16 + hn) * ROW + c];   // c == HD+1 sums the l's
+            }
+        }
+        part[(((size_t)t * H + g * QH + hn) * n_splits + split) * ROW + c] = acc;
+    }
+}
+
+template <int HD>
+__global__ void attn_decode_combine_kernel(const float* __restrict__ part, bf16* __restrict__ out, int H,
+                                           int n_splits) {
+    constexpr int ROW = HD + 2;
+    const int t = blockIdx.x, h = blockIdx.y;
+    const float* rec = part + ((size_t)t * H + h) * n_splits * ROW;
+    float M = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) M = fmaxf(M, rec[(size_t)s * ROW + HD]);
+    float L = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+        const float ms = rec[(size_t)s * ROW + HD];
+        L += (ms == -INFINITY) ? 0.f : exp2f(ms - M) * rec[(size_t)s * ROW + HD + 1];
+    }
+    const float inv = 1.0f / fmaxf(L, 1e-30f);
+    for (int c = threadIdx.x; c < HD; c += blockDim.x) {
+        float acc = 0.f;
+        for (int s = 0; s < n_splits; ++s) {
+            const float ms = rec[(size_t)s * ROW + HD];
+            if (ms != -INFINITY) acc += exp2f(ms - M) * rec[(size_t)s * ROW + c];
+        }
+        out[((size_t)t * H + h) * HD + c] = (bf16)(acc * inv);
+    }
+}
+
+// Bytes of fp32 scratch that a call needs.
+extern "C" size_t spite_attn_decode_workspace(int T, int H, int hd, int n_splits) {
+    return (size_t)T * H * n_splits * (hd + 2) * sizeof(float);
+}
+
+extern "C" int spite_attn_decode(const void* q, const void* k_pages, const void* v_pages, void* out, void* workspace,
+                                 const int* positions, const int* seq_of_token, const int* block_table,
+                                 int max_blocks, int T, int H, int G, int hd, int page_size, int vis, int span,
+                                 float scale, int n_splits, hipStream_t st) {
+    SP_REQUIRE(T >= 0 && H > 0 && G > 0 && H % G == 0, "attn_decode: %d query heads over %d kv heads", H, G);
+    SP_REQUIRE(H / G <= 16, "attn_decode: %d query heads per kv head, at most 16", H / G);
+    SP_REQUIRE(hd == 64 || hd == 128, "attn_decode: head size %d (this kernel has 64 and 128)", hd);
+    SP_REQUIRE(page_size > 0 && page_size % 32 == 0, "attn_decode: page size %d must be a multiple of 32", page_size);
+    SP_REQUIRE(max_blocks > 0 && n_splits >= 1 && n_splits <= 65535, "attn_decode: bad table width or split count");
+    SP_REQUIRE(vis == SP_VIS_FULL || span > 0, "attn_decode: chunk or window of %d", span);
+    SP_REQUIRE(G <= 65535 && T <= 65535, "attn_decode: too many heads or tokens for one launch");
+    if (T == 0) return 0;
+    const float sl = scale * 1.4426950408889634f;
+    dim3 grid(n_splits, G, T);
+    const size_t sh = (size_t)4 * 16 * (hd + 2) * sizeof(float);
+    if (hd == 128) {
+        attn_decode_kernel<128><<<grid, 256, sh, st>>>((const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages,
+            (float*)workspace, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, n_splits);
+        SP_LAUNCH_CHECK("attn_decode");
+        attn_decode_combine_kernel<128><<<dim3(T, H), 64, 0, st>>>((const float*)workspace, (bf16*)out, H, n_splits);
+    } else {
+        attn_decode_kernel<64><<<grid, 256, sh, st>>>((const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages,
+            (float*)workspace, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, n_splits);
+        SP_LAUNCH_CHECK("attn_decode");
+        attn_decode_combine_kernel<64><<<dim3(T, H), 64, 0, st>>>((const float*)workspace, (bf16*)out, H, n_splits);
+    }
+    SP_LAUNCH_CHECK("attn_decode_combine");
+    return 0;
+}

@@ -19,7 +19,7 @@ void attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
     extern __shared__ float smem[];
     float* q_sh = smem;                 // [hd]
     float* p_sh = smem + hd;            // [64]
-    long long* row_sh = (long long*)(p_sh + 64);   // [64] element offset of each key's row, -1 = none
+    long long* row_sh = (long long*)(p_sh + 64);   // [64] element offset of each key's value column, -1 = none
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int g = h / (H / G);
     const int p = positions[t];
@@ -43,8 +43,9 @@ void attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
             if (page < 0) {
                 s = NAN;   // a page that was given back is asked for: poison the result
             } else {
-                row = (((long long)page * G + g) * ps + (j % ps)) * hd;
-                const T* kr = k_pages + row;
+                const long long pg = (long long)page * G + g;
+                row = pg * hd * ps + (j % ps);            // value pages are [page][kv head][hd][offset]
+                const T* kr = k_pages + (pg * ps + (j % ps)) * hd;
                 float acc = 0.f;
                 for (int c = 0; c < hd; ++c) acc = fmaf(q_sh[c], to_f32<T>(kr[c]), acc);
                 s = acc * scale;
@@ -67,7 +68,7 @@ void attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
                 float acc = o[u] * alpha;
                 for (int jj = 0; jj < n_valid; ++jj) {
                     const long long r = row_sh[jj];
-                    const float vv = r >= 0 ? to_f32<T>(v_pages[r + c]) : 0.f;
+                    const float vv = r >= 0 ? to_f32<T>(v_pages[r + (long long)c * ps]) : 0.f;
                     acc = fmaf(p_sh[jj], vv, acc);
                 }
                 o[u] = acc;

@@ -86,8 +86,10 @@ extern "C" int spite_add_rmsnorm(float* h, const float* d1, const float* d2, con
 // the fused projection row.  Queries and keys: rotate by pos*inv_freq (if use_rope), then
 // the weightless RMS norm over the head (if use_norm); queries alone are then multiplied by
 // ln(floor((pos+1)/floor_scale)+1)*attn_scale+1 (if use_temp).  Keys and values go to the
-// request's page: cache row = slot_map[t] = page*page_size + offset, pages laid out
-// [page][kv head][offset][hd].
+// request's page: cache row = slot_map[t] = page*page_size + offset.  Key pages are laid out
+// [page][kv head][offset][hd]; value pages transposed, [page][kv head][hd][offset], so that
+// the attention kernels read eight consecutive keys of one value column in one load (the
+// layout of an MFMA operand whose sum runs over keys).
 #define SP_MAX_PAIRS 4   // head sizes up to 512
 template <typename T>
 __global__ void rope_kvwrite_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
@@ -114,11 +116,12 @@ __global__ void rope_kvwrite_kernel(const T* __restrict__ qkv, T* __restrict__ q
         if (slot < 0) return;
         const int g = is_v ? hh - H - G : hh - H;
         const size_t page = slot / ps, off = slot % ps;
-        dst = (is_v ? v_pages : k_pages) + ((page * G + g) * ps + off) * hd;
-    }
-    if (is_v) {
-        for (int c = lane; c < hd; c += 64) dst[c] = src[c];
-        return;
+        if (is_v) {
+            T* col = v_pages + (page * G + g) * hd * ps + off;
+            for (int c = lane; c < hd; c += 64) col[(size_t)c * ps] = src[c];
+            return;
+        }
+        dst = k_pages + ((page * G + g) * ps + off) * hd;
     }
     float x0[SP_MAX_PAIRS], x1[SP_MAX_PAIRS];
     float ss = 0.f;

@@ -1,0 +1,190 @@
+// Weight-streaming product for few rows (decode): Y[M,N] = X[M,K] . W[N,K]^T, bf16 in, fp32
+// accumulate on MFMA 16x16x32, for M up to a few dozen.  The time goes into reading W once
+// at HBM speed, so the shape of the kernel is the shape of that stream:
+//
+//  * A workgroup owns 16*R rows of W (R MFMA tiles) and all of K; its NW waves take the
+//    128-element blocks of K in turn (wave w: blocks w, w+NW, ...) and their partial sums
+//    meet in LDS.  Small N times large K still gives thousands of waves, each with several
+//    16-byte loads per lane in flight.
+//  * W is the MFMA "A" operand (rows of W = rows of the tile), X the "B" operand (tokens =
+//    columns).  MFMA does not care in which order k runs as long as both operands agree, so
+//    lane (row r, quarter q) reads 8*S consecutive elements W[r][kb + q*8S ..]: every row is
+//    read in runs of 64*S bytes.  (Plain loads: a 128-byte line is shared by two load
+//    instructions, and non-temporal loads were measured to fetch it twice.)
+//  * Grouped form (experts): see gemm_generic.hip.  A slot's scale multiplies the fp32 sums
+//    (W.(s x) = s (W.x)), so the scaled input is never rounded.  With GLU the workgroup also
+//    owns the matching "up" rows N+n and writes silu(gate) * up.
+//
+// A row's sum runs over k in an order that does not depend on M or on the other rows.
+#include "common.h"
+
+template <int R, int G, int S, int NW, bool GLU, typename TY>
+__global__ __launch_bounds__(NW * 64)
+void gemm_skinny_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restrict__ W, long w_group_stride,
+                        TY* __restrict__ Y, int ldy, int M, int N, int K,
+                        const int* __restrict__ offsets, int n_groups, const int* __restrict__ a_rows,
+                        const float* __restrict__ a_scale, const int* __restrict__ y_rows) {
+    constexpr int RA = GLU ? 2 * R : R;        // A tiles per wave
+    constexpr int KB = 32 * S;                 // k elements per block
+    constexpr int J = RA * G * 4;              // partial sums per lane
+    constexpr int MT = 16 * G;                 // slots per workgroup
+    extern __shared__ float red[];             // [NW][J][64]
+
+    int g = 0, row0, row_end = M;
+    if (offsets) {
+        int mt = blockIdx.y, acc = 0;
+        g = -1;
+        for (int e = 0; e < n_groups; ++e) {
+            const int b = offsets[e], en = offsets[e + 1];
+            const int nt = (en - b + MT - 1) / MT;
+            if (mt < acc + nt) { g = e; row0 = b + (mt - acc) * MT; row_end = en; break; }
+            acc += nt;
+        }
+        if (g < 0) return;
+    } else {
+        row0 = blockIdx.y * MT;
+        if (row0 >= M) return;
+    }
+    const int n0 = blockIdx.x * (16 * R);
+    const bf16* Wg = W + (size_t)g * w_group_stride;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, q = lane >> 4;
+
+    const bf16* wp[RA];
+#pragma unroll
+    for (int a = 0; a < RA; ++a) {
+        const int n = n0 + (a % R) * 16 + r;
+        const size_t row = (GLU && a >= R) ? (size_t)N + n : (size_t)n;
+        wp[a] = n < N ? Wg + row * K : nullptr;
+    }
+    const bf16* xp[G];
+#pragma unroll
+    for (int b = 0; b < G; ++b) {
+        const int s = row0 + b * 16 + r;
+        xp[b] = s < row_end ? X + (size_t)(a_rows ? a_rows[s] : s) * ldx : nullptr;
+    }
+
+    f32x4 acc[RA][G];
+#pragma unroll
+    for (int a = 0; a < RA; ++a)
+#pragma unroll
+        for (int b = 0; b < G; ++b) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    // Two register buffers, named apart so that every index is a constant: block i+1 is in
+    // flight while block i is multiplied.
+    bf16x8 wa0[RA][S], xb0[G][S], wa1[RA][S], xb1[G][S];
+    auto load = [&](bf16x8 (&wa)[RA][S], bf16x8 (&xb)[G][S], int kb) {
+#pragma unroll
+        for (int s = 0; s < S; ++s) {
+            const int k = kb + q * (8 * S) + s * 8;
+            const bool in = k < K;             // K is a multiple of 8
+#pragma unroll
+            for (int a = 0; a < RA; ++a)
+                wa[a][s] = (in && wp[a]) ? *(const bf16x8*)(wp[a] + k) : zero;
+#pragma unroll
+            for (int b = 0; b < G; ++b)
+                xb[b][s] = (in && xp[b]) ? *(const bf16x8*)(xp[b] + k) : zero;
+        }
+    };
+    auto mul = [&](bf16x8 (&wa)[RA][S], bf16x8 (&xb)[G][S]) {
+#pragma unroll
+        for (int s = 0; s < S; ++s)
+#pragma unroll
+            for (int a = 0; a < RA; ++a)
+#pragma unroll
+                for (int b = 0; b < G; ++b)
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[a][s], xb[b][s], acc[a][b], 0, 0, 0);
+    };
+    constexpr int STEP = NW * KB;
+    int kb = wave * KB;
+    if (kb < K) load(wa0, xb0, kb);
+    while (kb < K) {
+        if (kb + STEP < K) load(wa1, xb1, kb + STEP);
+        mul(wa0, xb0);
+        kb += STEP;
+        if (kb >= K) break;
+        if (kb + STEP < K) load(wa0, xb0, kb + STEP);
+        mul(wa1, xb1);
+        kb += STEP;
+    }
+
+    // partial sums of the waves meet in LDS: red[wave][j][lane]
+#pragma unroll
+    for (int a = 0; a < RA; ++a)
+#pragma unroll
+        for (int b = 0; b < G; ++b)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                red[(wave * J + (a * G + b) * 4 + i) * 64 + lane] = acc[a][b][i];
+    __syncthreads();
+    // acc[a][b][i] of lane (r, q) is the element (row n0 + a*16 + q*4 + i, slot row0 + b*16 + r)
+    constexpr int JO = R * G * 4;              // outputs per lane position (gate and up fold into one)
+    for (int o = threadIdx.x; o < JO * 64; o += NW * 64) {
+        const int j = o >> 6, l = o & 63;
+        const int a = j / (G * 4), b = (j / 4) % G, i = j & 3;
+        const int n = n0 + a * 16 + (l >> 4) * 4 + i;
+        const int s = row0 + b * 16 + (l & 15);
+        if (n >= N || s >= row_end) continue;
+        float v = 0.f, u = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            v += red[(w * J + j) * 64 + l];
+            if (GLU) u += red[(w * J + j + JO) * 64 + l];
+        }
+        if (a_scale) { const float sc = a_scale[s]; v *= sc; u *= sc; }
+        if (GLU) v = v / (1.0f + __expf(-v)) * u;
+        const size_t yr = y_rows ? (size_t)y_rows[s] : (size_t)s;
+        Y[yr * ldy + n] = from_f32<TY>(v);
+    }
+}
+
+template <int R, int G, int S, int NW>
+static int launch_skinny(const void* X, int ldx, const void* W, long wgs, void* Y, int y_dtype, int ldy, int M, int N,
+                         int K, const int* offsets, int n_groups, const int* a_rows, const float* a_scale,
+                         const int* y_rows, int glu, hipStream_t st) {
+    const int MT = 16 * G;
+    const int m_tiles = (M + MT - 1) / MT + (offsets ? n_groups : 0);
+    SP_REQUIRE(m_tiles <= 65535, "gemm_skinny: too many row tiles (%d)", m_tiles);
+    dim3 grid((N + 16 * R - 1) / (16 * R), m_tiles);
+    const size_t sh = (size_t)NW * (glu ? 2 : 1) * R * G * 4 * 64 * sizeof(float);
+#define SP_SK(GLUV, TY) do { \
+        auto kern = gemm_skinny_kernel<R, G, S, NW, GLUV, TY>; \
+        if (sh > 48 * 1024) { hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sh); \
+            if (e != hipSuccess) return sp_fail("gemm_skinny: cannot get %zu bytes of LDS: %s", sh, hipGetErrorString(e)); } \
+        kern<<<grid, NW * 64, sh, st>>>((const bf16*)X, ldx, (const bf16*)W, wgs, (TY*)Y, ldy, M, N, K, offsets, \
+                                        n_groups, a_rows, a_scale, y_rows); } while (0)
+    if (glu) { if (y_dtype == SP_BF16) SP_SK(true, bf16); else SP_SK(true, float); }
+    else { if (y_dtype == SP_BF16) SP_SK(false, bf16); else SP_SK(false, float); }
+#undef SP_SK
+    SP_LAUNCH_CHECK("gemm_skinny");
+    return 0;
+}
+
+// `max_rows`: the most rows any group brings (M itself for a plain product); picks how many
+// token columns a workgroup carries.
+extern "C" int spite_gemm_skinny(const void* X, int ldx, const void* W, long w_group_stride, void* Y, int y_dtype,
+                                 int ldy, int M, int N, int K, const int* offsets, int n_groups, const int* a_rows,
+                                 const float* a_scale, const int* y_rows, int glu, int max_rows, int variant,
+                                 hipStream_t st) {
+    SP_REQUIRE(M >= 0 && N > 0 && K > 0 && ldx >= K && ldy >= N, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
+    SP_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "gemm_skinny: K=%d and the row stride %d must be multiples of 8", K, ldx);
+    SP_REQUIRE(((uintptr_t)X & 15) == 0 && ((uintptr_t)W & 15) == 0, "gemm_skinny: operands must be 16-byte aligned");
+    SP_REQUIRE(y_dtype == SP_BF16 || y_dtype == SP_F32, "gemm_skinny: output dtype %d", y_dtype);
+    SP_REQUIRE(!offsets || n_groups > 0, "gemm_skinny: grouped call without groups");
+    if (M == 0) return 0;
+#define SP_ARGS X, ldx, W, w_group_stride, Y, y_dtype, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, st
+    if (variant == 0) variant = max_rows <= 16 ? ((size_t)N * K >= ((size_t)1 << 28) ? 7 : 8) : (max_rows <= 32 ? 2 : 3);
+    switch (variant) {
+        case 1: return launch_skinny<1, 1, 4, 8>(SP_ARGS);
+        case 2: return launch_skinny<2, 2, 2, 8>(SP_ARGS);
+        case 3: return launch_skinny<2, 4, 2, 4>(SP_ARGS);
+        case 4: return launch_skinny<2, 1, 4, 8>(SP_ARGS);
+        case 5: return launch_skinny<1, 1, 4, 4>(SP_ARGS);
+        case 6: return launch_skinny<1, 1, 2, 8>(SP_ARGS);
+        case 7: return launch_skinny<4, 1, 2, 8>(SP_ARGS);
+        case 8: return launch_skinny<2, 1, 2, 8>(SP_ARGS);
+        default: return sp_fail("gemm_skinny: unknown variant %d", variant);
+    }
+#undef SP_ARGS
+}

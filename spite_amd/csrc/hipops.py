@@ -41,6 +41,8 @@ def lib():
             "spite_gemm_generic": [P, I, P, L, I, P, I, I, I, I, I, P, I, P, P, P, I, P],
             "spite_attn_generic": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, P],
             "spite_sample_rows": [P, I, I, I, P, P, P, P],
+            "spite_gemm_skinny": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, I, P],
+            "spite_attn_decode": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, P],
         }
         for name, args in sigs.items():
             fn = getattr(l, name)
@@ -70,6 +72,14 @@ def _ptr(t, name, dtype=None, optional=False):
     if dtype is not None and t.dtype != dtype:
         raise KernelError(f"{name}: dtype {t.dtype}, expected {dtype}")
     return t.data_ptr()
+
+
+def _check_pages(k_pages, v_pages, G, page_size, hd, what):
+    """Key pages [n, G, page_size, hd]; value pages transposed, [n, G, hd, page_size]."""
+    if (tuple(k_pages.shape[1:]) != (G, page_size, hd) or tuple(v_pages.shape[1:]) != (G, hd, page_size)
+            or k_pages.shape[0] != v_pages.shape[0]):
+        raise KernelError(f"{what}: key pages {tuple(k_pages.shape)}, value pages {tuple(v_pages.shape)} for "
+                          f"G={G} page={page_size} hd={hd}")
 
 
 def _stream():
@@ -116,8 +126,8 @@ def add_rmsnorm(h, w, eps, out=None, out32=None, d1=None, d2=None, rows=None, n_
 def rope_kvwrite(qkv, q_out, k_pages, v_pages, positions, slot_map, inv_freq, H, G, hd, page_size, *,
                  use_rope, adjacent, use_norm, norm_eps, use_temp, floor_scale, attn_scale, write_kv=True):
     """Rotation, weightless qk-norm and temperature of the fused projection's rows; keys and
-    values go to their cache rows.  qkv [T,(H+2G)*hd]; q_out [T,H*hd]; pages
-    [n_pages, G, page_size, hd]."""
+    values go to their cache rows.  qkv [T,(H+2G)*hd]; q_out [T,H*hd]; key pages
+    [n_pages, G, page_size, hd], value pages [n_pages, G, hd, page_size]."""
     T = qkv.shape[0]
     if qkv.shape[1] != (H + 2 * G) * hd:
         raise KernelError(f"rope_kvwrite: qkv {tuple(qkv.shape)} for H={H} G={G} hd={hd}")
@@ -126,8 +136,7 @@ def rope_kvwrite(qkv, q_out, k_pages, v_pages, positions, slot_map, inv_freq, H,
     if write_kv:
         if slot_map.numel() < T:
             raise KernelError("rope_kvwrite: slot map too small")
-        if tuple(k_pages.shape[1:]) != (G, page_size, hd) or k_pages.shape != v_pages.shape:
-            raise KernelError(f"rope_kvwrite: pages {tuple(k_pages.shape)} for G={G} page={page_size} hd={hd}")
+        _check_pages(k_pages, v_pages, G, page_size, hd, "rope_kvwrite")
     if use_rope and inv_freq.numel() != hd // 2:
         raise KernelError("rope_kvwrite: frequency table does not match the head size")
     dt = qkv.dtype
@@ -208,8 +217,7 @@ def attn_generic(q, k_pages, v_pages, out, positions, seq_of_token, block_table,
     [T,H*hd]; block_table int32 [n_seqs, max_blocks]."""
     if q.numel() < T * H * hd or out.numel() < T * H * hd:
         raise KernelError("attention: q or out too small")
-    if tuple(k_pages.shape[1:]) != (G, page_size, hd) or k_pages.shape != v_pages.shape:
-        raise KernelError(f"attention: pages {tuple(k_pages.shape)} for G={G} page={page_size} hd={hd}")
+    _check_pages(k_pages, v_pages, G, page_size, hd, "attention")
     if block_table.dim() != 2 or positions.numel() < T or seq_of_token.numel() < T:
         raise KernelError("attention: metadata too small")
     dt = q.dtype
@@ -233,3 +241,63 @@ def sample_rows(logits, temperature, uniform, out, n_rows=None):
                                    _ptr(temperature, "temperature", torch.float32, True),
                                    _ptr(uniform, "uniform", torch.float32, True),
                                    _ptr(out, "out", torch.int32), _stream()), "sample")
+
+
+def _gemm_checks(a, w, y, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, what):
+    if a.shape[-1] != K or y.shape[-1] != N:
+        raise KernelError(f"{what}: a {tuple(a.shape)}, y {tuple(y.shape)} for N={N} K={K}")
+    rows_w = 2 * N if glu else N
+    if w.shape[-1] != K or w.shape[-2] != rows_w:
+        raise KernelError(f"{what}: weight {tuple(w.shape)} for N={N} K={K} glu={glu}")
+    groups_w = w.shape[0] if w.dim() == 3 else 1
+    if offsets is not None and (groups_w < n_groups or offsets.numel() < n_groups + 1):
+        raise KernelError(f"{what}: fewer weight groups or offsets than groups")
+    if a_rows is None and a.shape[0] < M:
+        raise KernelError(f"{what}: A has fewer rows than M")
+    if y_rows is None and y.shape[0] < M:
+        raise KernelError(f"{what}: Y has fewer rows than M")
+    for name, t in (("a_rows", a_rows), ("a_scale", a_scale), ("y_rows", y_rows)):
+        if t is not None and t.numel() < M:
+            raise KernelError(f"{what}: {name} shorter than M")
+    return rows_w
+
+
+def gemm_skinny(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None,
+                glu=False, max_rows=None, variant=0):
+    """Weight-streaming bf16 product for few rows (see gemm_skinny.hip); arguments as gemm_generic.
+    ``max_rows``: the most rows a group can bring (default M)."""
+    rows_w = _gemm_checks(a, w, y, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, "gemm_skinny")
+    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise KernelError(f"gemm_skinny: bfloat16 operands only, got {a.dtype} and {w.dtype}")
+    _check(lib().spite_gemm_skinny(
+        _ptr(a, "a"), a.stride(0), _ptr(w, "w"), rows_w * K, _ptr(y, "y"), dtype_code(y.dtype), y.stride(0),
+        M, N, K, _ptr(offsets, "offsets", torch.int32, True), n_groups, _ptr(a_rows, "a_rows", torch.int32, True),
+        _ptr(a_scale, "a_scale", torch.float32, True), _ptr(y_rows, "y_rows", torch.int32, True), int(glu),
+        int(max_rows if max_rows is not None else M), int(variant), _stream()), "gemm_skinny")
+
+
+def attn_decode_workspace(T, H, hd, n_splits) -> int:
+    """Bytes of scratch that attn_decode needs."""
+    return T * H * n_splits * (hd + 2) * 4
+
+
+def attn_decode(q, k_pages, v_pages, out, workspace, positions, seq_of_token, block_table, T, H, G, hd,
+                page_size, vis, span, scale, n_splits):
+    """Split-KV decode attention on MFMA (bf16; head sizes 64 and 128; pages of a multiple of 32
+    keys): every row of q is one query against its request's cache."""
+    if q.dtype != torch.bfloat16:
+        raise KernelError(f"attn_decode: bfloat16 only, got {q.dtype}")
+    if q.numel() < T * H * hd or out.numel() < T * H * hd:
+        raise KernelError("attn_decode: q or out too small")
+    _check_pages(k_pages, v_pages, G, page_size, hd, "attn_decode")
+    if block_table.dim() != 2 or positions.numel() < T or seq_of_token.numel() < T:
+        raise KernelError("attn_decode: metadata too small")
+    if workspace.numel() * workspace.element_size() < attn_decode_workspace(T, H, hd, n_splits):
+        raise KernelError("attn_decode: workspace too small")
+    dt = torch.bfloat16
+    _check(lib().spite_attn_decode(
+        _ptr(q, "q", dt), _ptr(k_pages, "k_pages", dt), _ptr(v_pages, "v_pages", dt), _ptr(out, "out", dt),
+        _ptr(workspace, "workspace"), _ptr(positions, "positions", torch.int32),
+        _ptr(seq_of_token, "seq_of_token", torch.int32), _ptr(block_table, "block_table", torch.int32),
+        block_table.shape[1], T, H, G, hd, page_size, VIS[vis], int(span or 0), float(scale), int(n_splits),
+        _stream()), "attn_decode")

@@ -75,8 +75,22 @@ class Attention(Mixer):
                             floor_scale=temp[0] if temp else 1, attn_scale=temp[1] if temp else 0.0,
                             write_kv=cache.write)
         o = ws.take((T, H * hd), x.dtype)
-        hipops.attn_generic(q, cache.k_pages, cache.v_pages, o, ctx.positions, ctx.seq_of_token,
-                            cache.block_table, T, H, G, hd, cache.page_size, self.visibility, self.span, self.scale)
+        if (ctx.decode_only and x.dtype == torch.bfloat16 and hd in (64, 128) and cache.page_size % 32 == 0
+                and H // G <= 16):
+            # split the longest request's keys so that about a thousand workgroups run
+            longest = int(ctx.host.starts.max()) + 1
+            if self.visibility != "full":
+                longest = min(longest, self.span)
+            blocks = -(-longest // 32)
+            n_splits = max(1, min(-(-1024 // (T * G)), -(-blocks // 4)))
+            scratch = ws.take((hipops.attn_decode_workspace(T, H, hd, n_splits) // 4,), torch.float32)
+            hipops.attn_decode(q, cache.k_pages, cache.v_pages, o, scratch, ctx.positions, ctx.seq_of_token,
+                               cache.block_table, T, H, G, hd, cache.page_size, self.visibility, self.span,
+                               self.scale, n_splits)
+        else:
+            hipops.attn_generic(q, cache.k_pages, cache.v_pages, o, ctx.positions, ctx.seq_of_token,
+                                cache.block_table, T, H, G, hd, cache.page_size, self.visibility, self.span,
+                                self.scale)
         out = ws.take((T, self.d), torch.float32)
         linear(o, self.wo, out)
         return out

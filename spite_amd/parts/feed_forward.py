@@ -92,10 +92,11 @@ class MoeTop1Sigmoid(FeedForward):
         offsets = ws.take((groups + 1,), torch.int32)
         hipops.moe_plan(expert, weight, src, scale, dst, offsets, T, E, self.fused_shared)
         act = ws.take((n, F), x.dtype)
-        linear(x, self.w_gate_up, act, glu=True, offsets=offsets, n_groups=groups, a_rows=src, a_scale=scale, rows=n)
+        linear(x, self.w_gate_up, act, glu=True, offsets=offsets, n_groups=groups, a_rows=src, a_scale=scale, rows=n,
+               max_rows=T)
         # slot s writes row dst[s]: rows [0,T) the routed result per token, rows [T,2T) the shared one
         y = ws.take((2 * T, d), torch.float32)
-        linear(act, self.w_down, y, offsets=offsets, n_groups=groups, y_rows=dst, rows=n)
+        linear(act, self.w_down, y, offsets=offsets, n_groups=groups, y_rows=dst, rows=n, max_rows=T)
         if self.fused_shared:
             return (y[:T], y[T:])
         act_s = ws.take((T, self.Fs), x.dtype)

@@ -17,13 +17,24 @@ def _widen(x):
     return y
 
 
-def linear(x, w, y, *, glu=False, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None, rows=None):
+SKINNY_MAX_ROWS = 64
+
+
+def linear(x, w, y, *, glu=False, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None, rows=None,
+           max_rows=None):
     """y[r] = W . x[r] for ``rows`` rows (default: all of x; for a row list: its length).
 
-    With ``glu`` the weight holds gate rows then up rows and y = silu(gate) * up."""
+    With ``glu`` the weight holds gate rows then up rows and y = silu(gate) * up.
+    ``max_rows``: the most rows that one group can bring (default: ``rows``)."""
     K = x.shape[-1]
     N = y.shape[-1]
     M = rows if rows is not None else x.shape[0]
+    most = max_rows if max_rows is not None else M
+    if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and most <= SKINNY_MAX_ROWS and K % 8 == 0
+            and x.stride(0) % 8 == 0):
+        hipops.gemm_skinny(x, w, y, M, N, K, offsets=offsets, n_groups=n_groups, a_rows=a_rows, a_scale=a_scale,
+                           y_rows=y_rows, glu=glu, max_rows=most)
+        return
     if w.dtype == torch.float32 and x.dtype != torch.float32:
         x32 = _widen(x)
         if y.dtype == torch.float32:

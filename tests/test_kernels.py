@@ -1,0 +1,326 @@
+"""Each kernel alone against a plain PyTorch reference in float64, at sizes other than the
+tiny models': widths and vocabularies that are no power of two, head sizes in steps of 8,
+any number of heads and groups, page edges."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import plain_llama4 as plain
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def ops():
+    from spite_amd.csrc import hipops
+    return hipops
+
+
+def rnd(*shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed + sum(shape))
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def tol_for(dtype, ref):
+    # fp32: accumulation noise; bf16: one rounding of the result (2^-9 relative) plus that
+    return (2e-5 if dtype == torch.float32 else 6e-3) * max(float(ref.abs().max()), 1e-6)
+
+
+# ------------------------------------------------------------------ embedding, norm
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embed(dtype):
+    table = rnd(301, 72, dtype=dtype)
+    ids = torch.tensor([0, 300, 17, 17, 5], dtype=torch.int32, device=DEV)
+    h = torch.empty(5, 72, dtype=torch.float32, device=DEV)
+    ops().embed(ids, table, h)
+    assert torch.equal(h, table[ids.long()].float())
+
+
+@pytest.mark.parametrize("d", [40, 96, 1000, 5120])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_add_rmsnorm(d, out_dtype):
+    T = 7
+    h, d1, d2, w = rnd(T, d), rnd(T, d, seed=1), rnd(T, d, seed=2), rnd(d, seed=3) + 1.0
+    ref_h = h.double() + d1.double() + d2.double()
+    ref = F.rms_norm(ref_h, (d,), w.double(), 1e-6)
+    out = torch.empty(T, d, dtype=out_dtype, device=DEV)
+    out32 = torch.empty(T, d, dtype=torch.float32, device=DEV)
+    hh = h.clone()
+    ops().add_rmsnorm(hh, w, 1e-6, out=out, out32=out32, d1=d1, d2=d2)
+    assert (hh.double() - ref_h).abs().max() < 1e-6
+    assert (out32.double() - ref).abs().max() < tol_for(torch.float32, ref)
+    assert (out.double() - ref).abs().max() < tol_for(out_dtype, ref)
+    # chosen rows only, h untouched
+    rows = torch.tensor([6, 2], dtype=torch.int32, device=DEV)
+    out2 = torch.empty(2, d, dtype=torch.float32, device=DEV)
+    hh = h.clone()
+    ops().add_rmsnorm(hh, w, 1e-6, out=out2, d1=d1, rows=rows, write_h=False)
+    ref2 = F.rms_norm(h.double() + d1.double(), (d,), w.double(), 1e-6)[[6, 2]]
+    assert torch.equal(hh, h) and (out2.double() - ref2).abs().max() < tol_for(torch.float32, ref2)
+
+
+# ------------------------------------------------------------------ rotation and cache write
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,G,hd,adjacent,norm,temp", [(4, 2, 16, False, True, False), (6, 3, 24, False, False, True),
+                                                       (5, 1, 64, True, True, True), (8, 8, 128, False, True, False),
+                                                       (2, 1, 256, False, True, False)])
+def test_rope_kvwrite(dtype, H, G, hd, adjacent, norm, temp):
+    T, ps, n_pages = 11, 4, 9
+    qkv = rnd(T, (H + 2 * G) * hd, dtype=dtype)
+    pos = torch.tensor([3, 4, 5, 0, 1, 2, 3, 40, 41, 42, 7], dtype=torch.int32, device=DEV)
+    slots = torch.tensor([5, 6, 7, 12, 13, 14, 15, 0, 1, 2, 35], dtype=torch.int32, device=DEV)
+    inv = plain.rope_inv_freq(hd, 10000.0, None).to(torch.float32).to(DEV)
+    q = torch.empty(T, H * hd, dtype=dtype, device=DEV)
+    kp = torch.zeros(n_pages, G, ps, hd, dtype=dtype, device=DEV)
+    vp = torch.zeros(n_pages, G, hd, ps, dtype=dtype, device=DEV)          # values are kept transposed
+    ops().rope_kvwrite(qkv, q, kp, vp, pos, slots, inv, H, G, hd, ps, use_rope=True, adjacent=adjacent, use_norm=norm,
+                       norm_eps=1e-5, use_temp=temp, floor_scale=4, attn_scale=0.1)
+    x = qkv.double().cpu()
+    qq, kk, vv = (x[:, :H * hd].view(T, H, hd), x[:, H * hd:(H + G) * hd].view(T, G, hd), x[:, (H + G) * hd:].view(T, G, hd))
+    pc = pos.cpu()
+    pairing = "adjacent" if adjacent else "half"
+    rq, rk = plain.apply_rope(qq, pc, inv.double().cpu(), pairing), plain.apply_rope(kk, pc, inv.double().cpu(), pairing)
+    if norm:
+        rq, rk = plain.qk_l2_norm(rq, 1e-5), plain.qk_l2_norm(rk, 1e-5)
+    if temp:
+        rq = rq * plain.attn_temperature(pc, 4, 0.1)[:, None, None]
+    tol = tol_for(dtype, rq) * (4 if dtype == torch.float32 else 1)
+    assert (q.double().cpu().view(T, H, hd) - rq).abs().max() < tol
+    for t in range(T):
+        page, off = int(slots[t]) // ps, int(slots[t]) % ps
+        assert (kp[page, :, off].double().cpu() - rk[t]).abs().max() < tol
+        assert torch.equal(vp[page, :, :, off].cpu().double(), vv[t])
+    written = {(int(s) // ps, int(s) % ps) for s in slots}
+    for p in range(n_pages):
+        for o in range(ps):
+            if (p, o) not in written:
+                assert float(kp[p, :, o].abs().sum()) == 0 and float(vp[p, :, :, o].abs().sum()) == 0
+
+
+def test_rope_kvwrite_refuses_odd_sizes():
+    from spite_amd.csrc.hipops import KernelError
+    z = torch.zeros(1, 3 * 15, device=DEV)
+    with pytest.raises(KernelError, match="even"):
+        ops().rope_kvwrite(z, torch.zeros(1, 15, device=DEV), torch.zeros(1, 1, 4, 15, device=DEV),
+                           torch.zeros(1, 1, 15, 4, device=DEV), torch.zeros(1, dtype=torch.int32, device=DEV),
+                           torch.zeros(1, dtype=torch.int32, device=DEV), None, 1, 1, 15, 4, use_rope=False,
+                           adjacent=False, use_norm=False, norm_eps=1e-5, use_temp=False, floor_scale=1, attn_scale=0.0)
+
+
+# ------------------------------------------------------------------ products
+def gemm_reference(a, w, M, N, K, offsets=None, a_rows=None, a_scale=None, y_rows=None, glu=False, n_out_rows=None):
+    a64, w64 = a.double().cpu(), w.double().cpu()
+    out = torch.zeros(n_out_rows or M, N, dtype=torch.float64)
+    groups = [(0, M, 0)] if offsets is None else [(int(offsets[g]), int(offsets[g + 1]), g) for g in range(len(offsets) - 1)]
+    for b, e, g in groups:
+        for s in range(b, e):
+            x = a64[int(a_rows[s]) if a_rows is not None else s]
+            if a_scale is not None:
+                x = x * float(a_scale[s])
+            wg = w64[g] if w64.dim() == 3 else w64
+            y = wg @ x
+            if glu:
+                y = F.silu(y[:N]) * y[N:]
+            out[int(y_rows[s]) if y_rows is not None else s] = y
+    return out
+
+
+GEMM_SHAPES = [(1, 48, 64), (7, 100, 264), (16, 130, 1032), (33, 96, 96), (64, 72, 520), (5, 202, 144)]
+
+
+def run_gemm(fn, dtype, out_dtype, M, N, K, glu=False, grouped=False, **kw):
+    E = 5 if grouped else 1
+    a = rnd(M + 3, K, dtype=dtype, scale=0.5)
+    w = rnd(*((E,) if grouped else ()), (2 * N if glu else N), K, dtype=dtype, seed=1, scale=0.5)
+    args = dict(glu=glu)
+    n_out = M
+    if grouped:
+        g = torch.Generator().manual_seed(M)
+        cuts = sorted(torch.randint(0, M + 1, (E - 1,), generator=g).tolist())
+        offsets = torch.tensor([0] + cuts + [M], dtype=torch.int32)
+        a_rows = torch.randint(0, M + 3, (M,), generator=g).to(torch.int32)
+        a_scale = torch.rand(M, generator=g) + 0.5
+        y_rows = torch.randperm(M + 2, generator=g)[:M].to(torch.int32)
+        n_out = M + 2
+        args.update(offsets=offsets.to(DEV), n_groups=E, a_rows=a_rows.to(DEV), a_scale=a_scale.to(DEV), y_rows=y_rows.to(DEV))
+        ref = gemm_reference(a, w, M, N, K, offsets, a_rows, a_scale, y_rows, glu, n_out)
+    else:
+        ref = gemm_reference(a, w, M, N, K, glu=glu)
+    y = torch.zeros(n_out, N, dtype=out_dtype, device=DEV)
+    fn(a, w, y, M, N, K, **args, **kw)
+    err = (y.double().cpu() - ref).abs().max()
+    assert err < tol_for(out_dtype, ref), (err, float(ref.abs().max()))
+
+
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+@pytest.mark.parametrize("dtype,out_dtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                             (torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("glu,grouped", [(False, False), (True, False), (False, True), (True, True)])
+def test_gemm_generic(M, N, K, dtype, out_dtype, glu, grouped):
+    if K % 8:
+        pytest.skip("shape list is shared with the MFMA kernels")
+    run_gemm(ops().gemm_generic, dtype, out_dtype, M, N, K, glu, grouped)
+
+
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES + [(3, 40, 8), (12, 16, 4104)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("glu,grouped", [(False, False), (True, False), (False, True), (True, True)])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7])
+def test_gemm_skinny(M, N, K, out_dtype, glu, grouped, variant):
+    run_gemm(ops().gemm_skinny, torch.bfloat16, out_dtype, M, N, K, glu, grouped, variant=variant)
+
+
+def test_gemm_skinny_refuses_what_it_cannot_do():
+    from spite_amd.csrc.hipops import KernelError
+    a, w, y = rnd(2, 12, dtype=torch.bfloat16), rnd(8, 12, dtype=torch.bfloat16), rnd(2, 8)
+    with pytest.raises(KernelError, match="multiples of 8"):
+        ops().gemm_skinny(a, w, y, 2, 8, 12)
+    with pytest.raises(KernelError, match="bfloat16"):
+        ops().gemm_skinny(a.float(), w.float(), y, 2, 8, 12)
+
+
+# ------------------------------------------------------------------ attention over the paged cache
+class PagedKV:
+    """Keys and values of a few requests scattered over shuffled pages."""
+
+    def __init__(self, lens, G, hd, ps, dtype, seed=0, extra_pages=3):
+        g = torch.Generator().manual_seed(seed)
+        self.lens, self.G, self.hd, self.ps = lens, G, hd, ps
+        self.k = [torch.randn(n, G, hd, generator=g).to(dtype) for n in lens]
+        self.v = [torch.randn(n, G, hd, generator=g).to(dtype) for n in lens]
+        blocks = [-(-n // ps) for n in lens]
+        n_pages = sum(blocks) + extra_pages
+        perm = torch.randperm(n_pages, generator=g).tolist()
+        self.tables, at = [], 0
+        for b in blocks:
+            self.tables.append(perm[at:at + b])
+            at += b
+        # unused rows hold large values: a kernel that reads beyond a request's keys shows it
+        self.kp = torch.full((n_pages, G, ps, hd), 50.0, dtype=dtype)
+        self.vp = torch.full((n_pages, G, hd, ps), -70.0, dtype=dtype)
+        for s, n in enumerate(lens):
+            for j in range(n):
+                pg, off = self.tables[s][j // ps], j % ps
+                self.kp[pg, :, off] = self.k[s][j]
+                self.vp[pg, :, :, off] = self.v[s][j]
+        width = max(blocks)
+        self.bt = torch.full((len(lens), width), -1, dtype=torch.int32)
+        for s, tab in enumerate(self.tables):
+            self.bt[s, :len(tab)] = torch.tensor(tab, dtype=torch.int32)
+
+    def drop_below(self, s, first_pos):
+        """Gives back the pages wholly below first_pos (their table entries become -1)."""
+        for b in range(first_pos // self.ps):
+            self.bt[s, b] = -1
+
+
+def attention_reference(kv, queries, qs, H, vis, span):
+    """queries: list of (request, position); qs [T,H,hd]."""
+    out = torch.zeros(len(queries), H, kv.hd, dtype=torch.float64)
+    for t, (s, p) in enumerate(queries):
+        pos = torch.arange(p + 1)
+        mask = plain.visible_mask(pos, vis, span)[p:p + 1]
+        out[t] = plain.attention(qs[t:t + 1].double(), kv.k[s][:p + 1].double(), kv.v[s][:p + 1].double(), mask)[0]
+    return out
+
+
+def run_attention(kind, dtype, H, G, hd, ps, lens, queries, vis, span, n_splits=3, seed=0, planted=None):
+    kv = PagedKV(lens, G, hd, ps, dtype, seed)
+    T = len(queries)
+    g = torch.Generator().manual_seed(seed + 1)
+    qs = torch.randn(T, H, hd, generator=g).to(dtype)
+    if planted is not None:                      # one far key that the query must find
+        t, s, j = planted
+        kv.k[s][j] = (qs[t, ::H // G] * 3.0).to(dtype)
+        pg, off = kv.tables[s][j // ps], j % ps
+        kv.kp[pg, :, off] = kv.k[s][j]
+    for s, first in enumerate([plain_first(vis, span, max([p for ss, p in queries if ss == s], default=0))
+                               for s in range(len(lens))]):
+        low = min([plain_first(vis, span, p) for ss, p in queries if ss == s], default=0)
+        kv.drop_below(s, low)
+    ref = attention_reference(kv, queries, qs, H, vis, span)
+    positions = torch.tensor([p for _, p in queries], dtype=torch.int32, device=DEV)
+    seq = torch.tensor([s for s, _ in queries], dtype=torch.int32, device=DEV)
+    out = torch.zeros(T, H * hd, dtype=dtype, device=DEV)
+    q_dev, kp, vp, bt = qs.reshape(T, H * hd).to(DEV), kv.kp.to(DEV), kv.vp.to(DEV), kv.bt.to(DEV)
+    scale = 1.0 / math.sqrt(hd)
+    if kind == "generic":
+        ops().attn_generic(q_dev, kp, vp, out, positions, seq, bt, T, H, G, hd, ps, vis, span, scale)
+    else:
+        wsz = ops().attn_decode_workspace(T, H, hd, n_splits)
+        scratch = torch.empty(wsz // 4, dtype=torch.float32, device=DEV)
+        ops().attn_decode(q_dev, kp, vp, out, scratch, positions, seq, bt, T, H, G, hd, ps, vis, span, scale, n_splits)
+    got = out.double().cpu().view(T, H, hd)
+    err = (got - ref).abs().max()
+    assert torch.isfinite(got).all()
+    # bf16: P is rounded as an MFMA operand and the output once
+    tol = 2e-5 if dtype == torch.float32 else 1.5e-2
+    assert err < tol * max(1.0, float(ref.abs().max())), err
+    return got, ref
+
+
+def plain_first(vis, span, p):
+    return {"full": 0, "chunk": (p // span) * span if span else 0, "window": max(p - span + 1, 0) if span else 0}[vis]
+
+
+ATT_CASES = [
+    # H, G, hd, page, lens, queries (request, position), visibility, span
+    (4, 2, 16, 4, [9, 30], [(0, 8), (1, 29), (1, 3), (0, 0)], "full", 0),
+    (6, 3, 24, 8, [70], [(0, 69), (0, 16), (0, 15), (0, 32)], "chunk", 16),
+    (6, 3, 24, 8, [70], [(0, 69), (0, 20), (0, 19), (0, 5)], "window", 20),
+    (5, 1, 64, 32, [200, 64], [(0, 199), (1, 63), (0, 64), (0, 31), (0, 32)], "full", 0),
+    (8, 2, 128, 64, [300], [(0, 299), (0, 255), (0, 256), (0, 128)], "chunk", 128),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", ATT_CASES, ids=lambda c: f"H{c[0]}G{c[1]}hd{c[2]}ps{c[3]}{c[6]}")
+def test_attn_generic(dtype, case):
+    H, G, hd, ps, lens, queries, vis, span = case
+    run_attention("generic", dtype, H, G, hd, ps, lens, queries, vis, span)
+
+
+DEC_CASES = [
+    (5, 1, 64, 32, [200, 64, 1], [(0, 199), (1, 63), (2, 0)], "full", 0),
+    (8, 2, 128, 64, [300, 129], [(0, 299), (1, 128)], "chunk", 128),
+    (40, 8, 128, 64, [1000, 33, 4096], [(0, 999), (1, 32), (2, 4095)], "full", 0),
+    (16, 1, 64, 32, [500], [(0, 499)], "window", 100),
+    (12, 4, 128, 32, [260, 70], [(0, 259), (1, 69)], "chunk", 64),
+]
+
+
+@pytest.mark.parametrize("n_splits", [1, 3, 16])
+@pytest.mark.parametrize("case", DEC_CASES, ids=lambda c: f"H{c[0]}G{c[1]}hd{c[2]}ps{c[3]}{c[6]}")
+def test_attn_decode(case, n_splits):
+    H, G, hd, ps, lens, queries, vis, span = case
+    run_attention("decode", torch.bfloat16, H, G, hd, ps, lens, queries, vis, span, n_splits)
+
+
+@pytest.mark.parametrize("kind", ["generic", "decode"])
+def test_attention_finds_one_far_key_among_thousands(kind):
+    # random keys give nearly uniform weights, which would hide a key that is skipped: one key
+    # far back matches the query, and the output must be close to that key's value
+    got, ref = run_attention(kind, torch.bfloat16, 8, 2, 128, 64, [3000], [(0, 2999)], "full", 0, n_splits=7,
+                             planted=(0, 0, 77))
+    # the reference itself puts nearly all the weight on key 77: its output is that key's value
+    kv = PagedKV([3000], 2, 128, 64, torch.bfloat16, 0)
+    assert (ref[0, 0] - kv.v[0][77][0].double()).abs().max() < 0.05
+    assert (got - ref).abs().max() < 2e-2
+
+
+@pytest.mark.parametrize("kind", ["generic", "decode"])
+def test_attention_refuses_what_it_cannot_do(kind):
+    from spite_amd.csrc.hipops import KernelError
+    z = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device=DEV)
+    i32 = lambda *s: torch.zeros(*s, dtype=torch.int32, device=DEV)
+    with pytest.raises(KernelError):
+        if kind == "generic":
+            ops().attn_generic(z(1, 6 * 16), z(1, 4, 8, 16), z(1, 4, 16, 8), z(1, 6 * 16), i32(1), i32(1), i32(1, 4),
+                               1, 6, 4, 16, 8, "full", 0, 0.25)        # 6 heads over 4 kv heads
+        else:
+            ops().attn_decode(z(1, 4 * 48), z(1, 2, 32, 48), z(1, 2, 48, 32), z(1, 4 * 48),
+                              torch.zeros(4096, device=DEV), i32(1), i32(1), i32(1, 4), 1, 4, 2, 48, 32, "full", 0,
+                              0.1, 1)                                    # head size 48
