@@ -37,31 +37,72 @@ extern "C" int spite_embed(const int* ids, const void* table, int dtype, float* 
 
 // ------------------------------------------------------------------ residual add + RMSNorm
 // v = h[r] + d1[r] + d2[r]; (h[r] = v); out[i] = v * 1/sqrt(mean(v^2)+eps) * w, r = rows ? rows[i] : i.
-template <typename TO>
-__global__ void add_rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ d1,
-                                   const float* __restrict__ d2, const float* __restrict__ w,
-                                   TO* __restrict__ out, float* __restrict__ out32,
-                                   const int* __restrict__ rows, int d, float eps, int write_h) {
-    __shared__ float red[4];
+// One workgroup of NT threads per row; a thread keeps its elements (groups of four, strided
+// by NT) in registers between the sum and the scaling, so the row is read once.  The sum's
+// order depends on the width alone.
+#define NORM_NT 512
+#define NORM_MAX_V 8     // widths up to 4*NT*MAX_V = 16384 stay in registers
+template <typename TO, bool VEC>
+__global__ __launch_bounds__(NORM_NT)
+void add_rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ d1,
+                        const float* __restrict__ d2, const float* __restrict__ w,
+                        TO* __restrict__ out, float* __restrict__ out32,
+                        const int* __restrict__ rows, int d, float eps, int write_h) {
+    __shared__ float red[NORM_NT / 64];
     const int i = blockIdx.x;
     const size_t r = rows ? (size_t)rows[i] : (size_t)i;
     float* hr = h + r * d;
     const float* a = d1 ? d1 + r * d : nullptr;
     const float* b = d2 ? d2 + r * d : nullptr;
     float ss = 0.f;
-    for (int c = threadIdx.x; c < d; c += 256) {
-        float v = hr[c];
-        if (a) v += a[c];
-        if (b) v += b[c];
-        if (write_h) hr[c] = v;
-        ss += v * v;
+    if (VEC) {
+        // d is a multiple of 4 and at most 4*NT*MAX_V
+        f32x4 v[NORM_MAX_V];
+        const int nv = d >> 2;
+#pragma unroll
+        for (int u = 0; u < NORM_MAX_V; ++u) {
+            const int c = threadIdx.x + u * NORM_NT;
+            if (c < nv) {
+                f32x4 x = ((const f32x4*)hr)[c];
+                if (a) x += ((const f32x4*)a)[c];
+                if (b) x += ((const f32x4*)b)[c];
+                if (write_h) ((f32x4*)hr)[c] = x;
+                v[u] = x;
+                ss += x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
+            }
+        }
+        const float ms = block_sum<NORM_NT>(ss, red) / (float)d;
+        const float scale = 1.0f / sqrtf(ms + eps);
+#pragma unroll
+        for (int u = 0; u < NORM_MAX_V; ++u) {
+            const int c = threadIdx.x + u * NORM_NT;
+            if (c < nv) {
+                const f32x4 ww = ((const f32x4*)w)[c];
+                f32x4 y;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) y[e] = v[u][e] * scale * ww[e];
+                if (out32) ((f32x4*)(out32 + (size_t)i * d))[c] = y;
+                if (out) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) out[(size_t)i * d + 4 * c + e] = from_f32<TO>(y[e]);
+                }
+            }
+        }
+        return;
     }
-    const float ms = block_sum<256>(ss, red) / (float)d;
+    for (int c = threadIdx.x; c < d; c += NORM_NT) {
+        float x = hr[c];
+        if (a) x += a[c];
+        if (b) x += b[c];
+        if (write_h) hr[c] = x;
+        ss += x * x;
+    }
+    const float ms = block_sum<NORM_NT>(ss, red) / (float)d;
     const float scale = 1.0f / sqrtf(ms + eps);
-    for (int c = threadIdx.x; c < d; c += 256) {
-        float v = hr[c];
-        if (!write_h) { if (a) v += a[c]; if (b) v += b[c]; }
-        const float y = v * scale * w[c];
+    for (int c = threadIdx.x; c < d; c += NORM_NT) {
+        float x = hr[c];
+        if (!write_h) { if (a) x += a[c]; if (b) x += b[c]; }
+        const float y = x * scale * w[c];
         if (out) out[(size_t)i * d + c] = from_f32<TO>(y);
         if (out32) out32[(size_t)i * d + c] = y;
     }
@@ -72,11 +113,14 @@ extern "C" int spite_add_rmsnorm(float* h, const float* d1, const float* d2, con
                                  float eps, int write_h, hipStream_t st) {
     SP_REQUIRE(n_rows >= 0 && d > 0 && eps > 0.f, "add_rmsnorm: bad sizes rows=%d d=%d eps=%g", n_rows, d, eps);
     if (n_rows == 0) return 0;
-    if (out_dtype == SP_F32)
-        add_rmsnorm_kernel<float><<<n_rows, 256, 0, st>>>(h, d1, d2, w, (float*)out, out32, rows, d, eps, write_h);
-    else if (out_dtype == SP_BF16)
-        add_rmsnorm_kernel<bf16><<<n_rows, 256, 0, st>>>(h, d1, d2, w, (bf16*)out, out32, rows, d, eps, write_h);
+    auto al = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
+    const bool vec = d % 4 == 0 && d <= 4 * NORM_NT * NORM_MAX_V && al(h) && al(d1) && al(d2) && al(w) && al(out32);
+#define SP_NORM(TO) do { if (vec) add_rmsnorm_kernel<TO, true><<<n_rows, NORM_NT, 0, st>>>(h, d1, d2, w, (TO*)out, out32, rows, d, eps, write_h); \
+        else add_rmsnorm_kernel<TO, false><<<n_rows, NORM_NT, 0, st>>>(h, d1, d2, w, (TO*)out, out32, rows, d, eps, write_h); } while (0)
+    if (out_dtype == SP_F32) SP_NORM(float);
+    else if (out_dtype == SP_BF16) SP_NORM(bf16);
     else return sp_fail("add_rmsnorm: unknown dtype %d", out_dtype);
+#undef SP_NORM
     SP_LAUNCH_CHECK("add_rmsnorm");
     return 0;
 }
@@ -192,24 +236,44 @@ extern "C" int spite_rope_kvwrite(const void* qkv, void* q_out, void* k_pages, v
 }
 
 // ------------------------------------------------------------------ top-1 sigmoid router
-// One wave per token: logits = W_r . x in fp32, the largest logit wins and the lowest index
-// wins a tie, weight = 1/(1+exp(-logit)).
-__global__ void router_top1_kernel(const float* __restrict__ x, const float* __restrict__ wr,
-                                   int* __restrict__ expert, float* __restrict__ weight,
-                                   float* __restrict__ logits_out, int d, int E) {
+// One workgroup per token: logits = W_r . x in fp32, the largest logit wins and the lowest
+// index wins a tie, weight = 1/(1+exp(-logit)).  The token's row sits in LDS; the waves take
+// the experts in turn, a lane's loads are independent 16-byte reads.  A logit's sum runs in
+// an order that depends on the width alone.
+#define ROUTER_NT 256
+__global__ __launch_bounds__(ROUTER_NT)
+void router_top1_kernel(const float* __restrict__ x, const float* __restrict__ wr,
+                        int* __restrict__ expert, float* __restrict__ weight,
+                        float* __restrict__ logits_out, int d, int E) {
+    extern __shared__ float xs[];            // [d] then [E] logits
+    float* lg = xs + d;
     const int t = blockIdx.x;
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float* xr = x + (size_t)t * d;
-    float best = 0.f; int best_e = -1;
-    for (int e = 0; e < E; ++e) {
+    for (int c = threadIdx.x; c < d; c += ROUTER_NT) xs[c] = xr[c];
+    __syncthreads();
+    const bool vec = (d & 3) == 0 && (((uintptr_t)wr) & 15) == 0;
+    for (int e = wave; e < E; e += ROUTER_NT / 64) {
         const float* w = wr + (size_t)e * d;
         float acc = 0.f;
-        for (int c = lane; c < d; c += 64) acc += w[c] * xr[c];
+        if (vec) {
+            const int nv = d >> 2;
+            for (int c = lane; c < nv; c += 64) {
+                const f32x4 ww = ((const f32x4*)w)[c];
+                const f32x4 xx = ((const f32x4*)xs)[c];
+                acc += ww[0] * xx[0] + ww[1] * xx[1] + ww[2] * xx[2] + ww[3] * xx[3];
+            }
+        } else {
+            for (int c = lane; c < d; c += 64) acc += w[c] * xs[c];
+        }
         acc = wave_sum(acc);
-        if (logits_out && lane == 0) logits_out[(size_t)t * E + e] = acc;
-        if (best_e < 0 || acc > best) { best = acc; best_e = e; }
+        if (lane == 0) lg[e] = acc;
     }
-    if (lane == 0) {
+    __syncthreads();
+    if (logits_out) for (int e = threadIdx.x; e < E; e += ROUTER_NT) logits_out[(size_t)t * E + e] = lg[e];
+    if (threadIdx.x == 0) {
+        float best = lg[0]; int best_e = 0;
+        for (int e = 1; e < E; ++e) if (lg[e] > best) { best = lg[e]; best_e = e; }
         expert[t] = best_e;
         weight[t] = 1.0f / (1.0f + expf(-best));
     }
@@ -218,8 +282,10 @@ __global__ void router_top1_kernel(const float* __restrict__ x, const float* __r
 extern "C" int spite_router_top1(const float* x, const float* wr, int* expert, float* weight,
                                  float* logits_out, int T, int d, int E, hipStream_t st) {
     SP_REQUIRE(T >= 0 && d > 0 && E > 0, "router: bad sizes T=%d d=%d E=%d", T, d, E);
+    const size_t sh = (size_t)(d + E) * sizeof(float);
+    SP_REQUIRE(sh <= 48 * 1024, "router: width %d with %d experts does not fit the kernel's LDS", d, E);
     if (T == 0) return 0;
-    router_top1_kernel<<<T, 64, 0, st>>>(x, wr, expert, weight, logits_out, d, E);
+    router_top1_kernel<<<T, ROUTER_NT, sh, st>>>(x, wr, expert, weight, logits_out, d, E);
     SP_LAUNCH_CHECK("router_top1");
     return 0;
 }

@@ -53,15 +53,21 @@ void gemm_skinny_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restr
     const bf16* wp[RA];
 #pragma unroll
     for (int a = 0; a < RA; ++a) {
-        const int n = n0 + (a % R) * 16 + r;
+        // rows past N read row N-1 again, slots past the group its last slot: the loads of
+        // the main loop carry no condition (a select on a loaded value would make the wave
+        // wait for it at once), lanes with one address are served by one request, and what
+        // such rows produce is never stored
+        int n = n0 + (a % R) * 16 + r;
+        n = n < N ? n : N - 1;
         const size_t row = (GLU && a >= R) ? (size_t)N + n : (size_t)n;
-        wp[a] = n < N ? Wg + row * K : nullptr;
+        wp[a] = Wg + row * K;
     }
     const bf16* xp[G];
 #pragma unroll
     for (int b = 0; b < G; ++b) {
-        const int s = row0 + b * 16 + r;
-        xp[b] = s < row_end ? X + (size_t)(a_rows ? a_rows[s] : s) * ldx : nullptr;
+        int s = row0 + b * 16 + r;
+        s = s < row_end ? s : row_end - 1;
+        xp[b] = X + (size_t)(a_rows ? a_rows[s] : s) * ldx;
     }
 
     f32x4 acc[RA][G];
@@ -78,13 +84,21 @@ void gemm_skinny_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restr
 #pragma unroll
         for (int s = 0; s < S; ++s) {
             const int k = kb + q * (8 * S) + s * 8;
-            const bool in = k < K;             // K is a multiple of 8
 #pragma unroll
-            for (int a = 0; a < RA; ++a)
-                wa[a][s] = (in && wp[a]) ? *(const bf16x8*)(wp[a] + k) : zero;
+            for (int a = 0; a < RA; ++a) wa[a][s] = *(const bf16x8*)(wp[a] + k);
 #pragma unroll
-            for (int b = 0; b < G; ++b)
-                xb[b][s] = (in && xp[b]) ? *(const bf16x8*)(xp[b] + k) : zero;
+            for (int b = 0; b < G; ++b) xb[b][s] = *(const bf16x8*)(xp[b] + k);
+        }
+    };
+    // the last block when K is no multiple of the block: chunks past K are zero (K % 8 == 0)
+    auto load_tail = [&](bf16x8 (&wa)[RA][S], bf16x8 (&xb)[G][S], int kb) {
+#pragma unroll
+        for (int s = 0; s < S; ++s) {
+            const int k = kb + q * (8 * S) + s * 8;
+#pragma unroll
+            for (int a = 0; a < RA; ++a) wa[a][s] = k < K ? *(const bf16x8*)(wp[a] + k) : zero;
+#pragma unroll
+            for (int b = 0; b < G; ++b) xb[b][s] = k < K ? *(const bf16x8*)(xp[b] + k) : zero;
         }
     };
     auto mul = [&](bf16x8 (&wa)[RA][S], bf16x8 (&xb)[G][S]) {
@@ -97,16 +111,21 @@ void gemm_skinny_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restr
                     acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[a][s], xb[b][s], acc[a][b], 0, 0, 0);
     };
     constexpr int STEP = NW * KB;
+    const int k_full = K / KB * KB;            // whole blocks end here
     int kb = wave * KB;
-    if (kb < K) load(wa0, xb0, kb);
-    while (kb < K) {
-        if (kb + STEP < K) load(wa1, xb1, kb + STEP);
+    if (kb < k_full) load(wa0, xb0, kb);
+    while (kb < k_full) {
+        if (kb + STEP < k_full) load(wa1, xb1, kb + STEP);
         mul(wa0, xb0);
         kb += STEP;
-        if (kb >= K) break;
-        if (kb + STEP < K) load(wa0, xb0, kb + STEP);
+        if (kb >= k_full) break;
+        if (kb + STEP < k_full) load(wa0, xb0, kb + STEP);
         mul(wa1, xb1);
         kb += STEP;
+    }
+    if (k_full < K && wave == (k_full / KB) % NW) {   // the partial block goes to the wave whose turn it is
+        load_tail(wa0, xb0, k_full);
+        mul(wa0, xb0);
     }
 
     // partial sums of the waves meet in LDS: red[wave][j][lane]
@@ -174,7 +193,12 @@ extern "C" int spite_gemm_skinny(const void* X, int ldx, const void* W, long w_g
     SP_REQUIRE(!offsets || n_groups > 0, "gemm_skinny: grouped call without groups");
     if (M == 0) return 0;
 #define SP_ARGS X, ldx, W, w_group_stride, Y, y_dtype, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, st
-    if (variant == 0) variant = max_rows <= 16 ? ((size_t)N * K >= ((size_t)1 << 28) ? 7 : 8) : (max_rows <= 32 ? 2 : 3);
+    // measured on MI355X (GB/s of W at Llama 4 Scout's shapes): one row tile per workgroup for
+    // the experts' grouped stream, two for the dense projections, four for the output matrix
+    if (variant == 0) {
+        if (max_rows <= 16) variant = offsets ? 6 : ((size_t)N * K >= ((size_t)1 << 28) ? 7 : 2);
+        else variant = max_rows <= 32 ? 2 : 3;
+    }
     switch (variant) {
         case 1: return launch_skinny<1, 1, 4, 8>(SP_ARGS);
         case 2: return launch_skinny<2, 2, 2, 8>(SP_ARGS);

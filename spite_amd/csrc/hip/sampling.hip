@@ -40,8 +40,10 @@ void sample_rows_kernel(const float* __restrict__ logits, int ld, int V, const f
     const int per = (V + SAMP_NT - 1) / SAMP_NT;
     const int b = tid * per, e = (b + per < V) ? b + per : V;
 
+    // arg-max: neighbouring threads read neighbouring elements; a thread meets its indices in
+    // rising order, so "greater than" keeps the lowest index of equal values
     float bv = 0.f; int bi = -1;
-    for (int i = b; i < e; ++i) {
+    for (int i = tid; i < V; i += SAMP_NT) {
         const float x = row[i];
         if (bi < 0 || x > bv) { bv = x; bi = i; }
     }

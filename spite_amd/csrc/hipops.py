@@ -43,6 +43,7 @@ def lib():
             "spite_sample_rows": [P, I, I, I, P, P, P, P],
             "spite_gemm_skinny": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, I, P],
             "spite_attn_decode": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, P],
+            "spite_gemm_mfma": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, P],
         }
         for name, args in sigs.items():
             fn = getattr(l, name)
@@ -301,3 +302,15 @@ def attn_decode(q, k_pages, v_pages, out, workspace, positions, seq_of_token, bl
         _ptr(seq_of_token, "seq_of_token", torch.int32), _ptr(block_table, "block_table", torch.int32),
         block_table.shape[1], T, H, G, hd, page_size, VIS[vis], int(span or 0), float(scale), int(n_splits),
         _stream()), "attn_decode")
+
+
+def gemm_mfma(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None, glu=False):
+    """Tiled bf16 MFMA product for many rows (see gemm_mfma.hip); arguments as gemm_generic."""
+    rows_w = _gemm_checks(a, w, y, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, "gemm_mfma")
+    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise KernelError(f"gemm_mfma: bfloat16 operands only, got {a.dtype} and {w.dtype}")
+    _check(lib().spite_gemm_mfma(
+        _ptr(a, "a"), a.stride(0), _ptr(w, "w"), rows_w * K, _ptr(y, "y"), dtype_code(y.dtype), y.stride(0),
+        M, N, K, _ptr(offsets, "offsets", torch.int32, True), n_groups, _ptr(a_rows, "a_rows", torch.int32, True),
+        _ptr(a_scale, "a_scale", torch.float32, True), _ptr(y_rows, "y_rows", torch.int32, True), int(glu),
+        _stream()), "gemm_mfma")

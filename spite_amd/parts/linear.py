@@ -30,10 +30,13 @@ def linear(x, w, y, *, glu=False, offsets=None, n_groups=1, a_rows=None, a_scale
     N = y.shape[-1]
     M = rows if rows is not None else x.shape[0]
     most = max_rows if max_rows is not None else M
-    if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and most <= SKINNY_MAX_ROWS and K % 8 == 0
-            and x.stride(0) % 8 == 0):
-        hipops.gemm_skinny(x, w, y, M, N, K, offsets=offsets, n_groups=n_groups, a_rows=a_rows, a_scale=a_scale,
-                           y_rows=y_rows, glu=glu, max_rows=most)
+    if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and K % 8 == 0 and x.stride(0) % 8 == 0:
+        if most <= SKINNY_MAX_ROWS:      # few rows: the time is the weights' stream
+            hipops.gemm_skinny(x, w, y, M, N, K, offsets=offsets, n_groups=n_groups, a_rows=a_rows,
+                               a_scale=a_scale, y_rows=y_rows, glu=glu, max_rows=most)
+        else:
+            hipops.gemm_mfma(x, w, y, M, N, K, offsets=offsets, n_groups=n_groups, a_rows=a_rows, a_scale=a_scale,
+                             y_rows=y_rows, glu=glu)
         return
     if w.dtype == torch.float32 and x.dtype != torch.float32:
         x32 = _widen(x)

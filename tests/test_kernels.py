@@ -173,6 +173,13 @@ def test_gemm_skinny(M, N, K, out_dtype, glu, grouped, variant):
     run_gemm(ops().gemm_skinny, torch.bfloat16, out_dtype, M, N, K, glu, grouped, variant=variant)
 
 
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES + [(200, 300, 264), (128, 128, 64), (130, 70, 1032), (257, 129, 72)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("glu,grouped", [(False, False), (True, False), (False, True), (True, True)])
+def test_gemm_mfma(M, N, K, out_dtype, glu, grouped):
+    run_gemm(ops().gemm_mfma, torch.bfloat16, out_dtype, M, N, K, glu, grouped)
+
+
 def test_gemm_skinny_refuses_what_it_cannot_do():
     from spite_amd.csrc.hipops import KernelError
     a, w, y = rnd(2, 12, dtype=torch.bfloat16), rnd(8, 12, dtype=torch.bfloat16), rnd(2, 8)
