@@ -306,6 +306,46 @@ def test_attn_decode(case, n_splits):
     run_attention("decode", torch.bfloat16, H, G, hd, ps, lens, queries, vis, span, n_splits)
 
 
+PORTION_CASES = [
+    # H, G, hd, page, cached lengths after the step, portions (request, first position, count), visibility, span
+    (5, 1, 64, 32, [200, 70, 1], [(0, 120, 80), (1, 0, 70), (2, 0, 1)], "full", 0),
+    (8, 2, 128, 64, [300], [(0, 0, 300)], "chunk", 128),
+    (8, 2, 128, 64, [300, 40], [(0, 250, 50), (1, 39, 1)], "chunk", 128),       # a portion across a chunk border
+    (40, 8, 128, 64, [130, 65], [(0, 97, 33), (1, 0, 65)], "full", 0),
+    (16, 1, 64, 32, [500], [(0, 380, 120)], "window", 100),
+    (12, 4, 128, 32, [260, 70], [(0, 258, 2), (1, 0, 70)], "chunk", 64),
+]
+
+
+@pytest.mark.parametrize("case", PORTION_CASES, ids=lambda c: f"H{c[0]}G{c[1]}hd{c[2]}ps{c[3]}{c[6]}")
+def test_attn_prefill(case):
+    H, G, hd, ps, lens, portions, vis, span = case
+    dtype = torch.bfloat16
+    kv = PagedKV(lens, G, hd, ps, dtype, seed=3)
+    queries = [(s, p) for s, first, count in portions for p in range(first, first + count)]
+    T = len(queries)
+    g = torch.Generator().manual_seed(4)
+    qs = torch.randn(T, H, hd, generator=g).to(dtype)
+    for s, first, count in portions:
+        kv.drop_below(s, plain_first(vis, span, first))
+    ref = attention_reference(kv, queries, qs, H, vis, span)
+    positions = torch.tensor([p for _, p in queries], dtype=torch.int32, device=DEV)
+    seq = torch.tensor([i for i, (s, first, count) in enumerate(portions) for _ in range(count)], dtype=torch.int32, device=DEV)
+    cu = [0]
+    for _, _, count in portions:
+        cu.append(cu[-1] + count)
+    tiles = [cu[i] + q0 for i, (_, _, count) in enumerate(portions) for q0 in range(0, count, 32)]
+    bt = torch.stack([kv.bt[s] for s, _, _ in portions]).to(DEV)
+    out = torch.zeros(T, H * hd, dtype=dtype, device=DEV)
+    ops().attn_prefill(qs.reshape(T, H * hd).to(DEV), kv.kp.to(DEV), kv.vp.to(DEV), out, positions, seq,
+                       torch.tensor(cu, dtype=torch.int32, device=DEV), bt,
+                       torch.tensor(tiles, dtype=torch.int32, device=DEV), len(tiles), H, G, hd, ps, vis, span,
+                       1.0 / math.sqrt(hd))
+    got = out.double().cpu().view(T, H, hd)
+    assert torch.isfinite(got).all()
+    assert (got - ref).abs().max() < 1.5e-2 * max(1.0, float(ref.abs().max()))
+
+
 @pytest.mark.parametrize("kind", ["generic", "decode"])
 def test_attention_finds_one_far_key_among_thousands(kind):
     # random keys give nearly uniform weights, which would hide a key that is skipped: one key
