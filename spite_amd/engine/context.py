@@ -28,11 +28,13 @@ class Workspace:
         self.device = device
         self._chunks = [torch.empty(max(nbytes, self.ALIGN), dtype=torch.uint8, device=device)]
         self._off = 0
+        self.generation = 0          # counts reallocations: addresses handed out earlier are stale after one
 
     def reset(self):
         if len(self._chunks) > 1:
             total = sum(c.numel() for c in self._chunks)
             self._chunks = [torch.empty(total, dtype=torch.uint8, device=self.device)]
+            self.generation += 1
         self._off = 0
 
     def take(self, shape, dtype) -> torch.Tensor:
@@ -44,8 +46,11 @@ class Workspace:
         cur = self._chunks[-1]
         start = (self._off + self.ALIGN - 1) // self.ALIGN * self.ALIGN
         if start + nbytes > cur.numel():
+            if torch.cuda.is_current_stream_capturing():
+                raise RuntimeError("workspace would grow while a graph is captured; warm the step up first")
             cur = torch.empty(max(nbytes + self.ALIGN, 2 * cur.numel()), dtype=torch.uint8, device=self.device)
             self._chunks.append(cur)
+            self.generation += 1
             start = 0
         self._off = start + nbytes
         if n == 0:

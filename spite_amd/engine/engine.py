@@ -53,10 +53,12 @@ class StepMeta:
         np.cumsum(counts, out=cu[1:])
         T = int(cu[-1])
         n_groups = cache.n_groups()
+        # table width: the next power of two, so that the shape of a step changes rarely
         widths = []
         for g in range(n_groups):
             w = max([cache.table_len(int(s), g) for s in slots], default=1)
-            widths.append(max(4, (w + 3) // 4 * 4))
+            widths.append(max(4, 1 << (w - 1).bit_length()))
+        self.widths = tuple(widths)
         rows = []
         for i, e in enumerate(entries):
             for w in e.want:
@@ -113,11 +115,15 @@ class Engine:
     def __init__(self, model: Union[str, dict, None] = None, *, dtype: str = "bfloat16", page_size: int = 64,
                  num_pages=None, cache_tokens: Optional[int] = None, max_batch_tokens: int = 2048,
                  max_requests: int = 8, device: str = "cuda:0", random_weights: bool = False, seed: int = 0,
-                 init_std: float = 0.02, spec: Optional[ModelSpec] = None, tensors: Optional[dict] = None):
+                 init_std: float = 0.02, spec: Optional[ModelSpec] = None, tensors: Optional[dict] = None,
+                 graphs: bool = True):
         """``model``: a folder with config.json and model.safetensors; with ``random_weights`` a
         folder, a config.json path or a config dict whose weights are drawn on the GPU from
         ``seed``.  ``spec`` (+ ``tensors`` by checkpoint name, or ``random_weights``) builds a
-        model from parts directly, without an architecture."""
+        model from parts directly, without an architecture.  With ``graphs`` a decode step (one
+        token of every request, every logit wanted) is captured in a HIP graph the second time
+        its shape comes up and replayed from then on: the step is bound by kernel launches
+        otherwise.  The graph holds the same kernels on the same buffers as the eager step."""
         if dtype not in _DTYPES:
             raise EngineError(f"dtype {dtype!r} (known: bfloat16, float32)")
         if not torch.cuda.is_available():
@@ -156,6 +162,10 @@ class Engine:
         self._pin_event = None
         self._meta_dev = None
         self.steps_run = 0
+        self.use_graphs = bool(graphs)
+        self._graphs: Dict[tuple, object] = {}     # shape of a decode step -> (graph, logits) or "seen"
+        self._graph_stamp = None
+        self.graph_replays = 0
 
     # ------------------------------------------------------------------ weights
     def _load_from_dict(self, tensors: Dict[str, torch.Tensor], ckpt_dtype):
@@ -259,12 +269,64 @@ class Engine:
         meta = StepMeta(self, entries)
         if trace is not None:
             meta.ctx.extras["trace"] = trace
-        self._step_ws.reset()
-        logits = self.model.forward(meta.ctx, self.cache, meta, self._arenas, self._step_ws)
+        logits = None
+        key = None
+        if (self.use_graphs and trace is None and meta.ctx.decode_only and meta.ctx.n_out == meta.ctx.n_seqs
+                and all(tuple(e.want) == (0,) for e in entries)):
+            key = (meta.ctx.n_seqs, meta.widths)
+            logits = self._replay(key)
+        if logits is None:
+            self._step_ws.reset()
+            if key is not None and self._graphs.get(key) == "seen":
+                logits = self._capture(key, meta)
+            else:
+                logits = self.model.forward(meta.ctx, self.cache, meta, self._arenas, self._step_ws)
+                if key is not None:
+                    self._graphs[key] = "seen"
+                    self._graph_stamp = self._stamp()
         if commit:
             for e in entries:
                 self.cache.commit(e.slot, len(e.tokens))
         self.steps_run += 1
+        return logits
+
+    # ------------------------------------------------------------------ graphs of decode steps
+    def _stamp(self):
+        """Changes whenever a buffer that graphs point into has been allocated anew."""
+        return (self._meta_dev.data_ptr() if self._meta_dev is not None else 0, self._step_ws.generation,
+                self._arenas[0].generation, self._arenas[1].generation)
+
+    def _replay(self, key):
+        if self._graph_stamp != self._stamp():
+            self._graphs.clear()           # their addresses are stale
+            self._graph_stamp = self._stamp()
+            return None
+        hit = self._graphs.get(key)
+        if hit is None or hit == "seen":
+            return None
+        graph, logits = hit
+        graph.replay()
+        self.graph_replays += 1
+        return logits
+
+    def _capture(self, key, meta):
+        for ws in self._arenas:
+            ws.reset()                     # merge what the warm-up step added, outside the capture
+        graph = torch.cuda.CUDAGraph()
+        try:
+            with torch.cuda.graph(graph):
+                logits = self.model.forward(meta.ctx, self.cache, meta, self._arenas, self._step_ws)
+        except Exception:
+            self._graphs.pop(key, None)
+            self.use_graphs = False        # fall back to eager steps for good, loudly
+            import warnings
+            warnings.warn("capturing the decode step in a HIP graph failed; steps run eagerly from now on")
+            self._step_ws.reset()
+            return self.model.forward(meta.ctx, self.cache, meta, self._arenas, self._step_ws)
+        graph.replay()                     # the capture itself computed nothing
+        self._graphs[key] = (graph, logits)
+        self._graph_stamp = self._stamp()
+        self.graph_replays += 1
         return logits
 
     def commit(self, entries: Sequence[StepEntry]) -> None:
