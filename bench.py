@@ -80,6 +80,7 @@ def main() -> int:
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--tiny", action="store_true", help="a small model of the same kind, to try the script")
+    ap.add_argument("--no-graphs", action="store_true", help="run decode steps eagerly (for kernel traces)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not measured")
@@ -103,7 +104,8 @@ def main() -> int:
     log(f"building {L} of {layers_full} layers, cache for {cache_tokens} positions")
     t0 = time.time()
     eng = Engine(cfg, dtype=args.dtype, page_size=page, cache_tokens=cache_tokens, max_requests=max_b,
-                 max_batch_tokens=max(args.prefill_tokens, max_b), random_weights=True, seed=0)
+                 max_batch_tokens=max(args.prefill_tokens, max_b), random_weights=True, seed=0,
+                 graphs=not args.no_graphs)
     torch.cuda.synchronize()
     log(f"model and cache on the GPU in {time.time() - t0:.1f} s, "
         f"{torch.cuda.memory_allocated() / 2**30:.1f} GiB allocated")

@@ -146,27 +146,41 @@ void attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_p
 }
 
 template <int HD>
-__global__ void attn_decode_combine_kernel(const float* __restrict__ part, bf16* __restrict__ out, int H,
-                                           int n_splits) {
+__global__ __launch_bounds__(HD)
+void attn_decode_combine_kernel(const float* __restrict__ part, bf16* __restrict__ out, int H, int n_splits) {
     constexpr int ROW = HD + 2;
-    const int t = blockIdx.x, h = blockIdx.y;
+    __shared__ float wsh[256];          // weight of every split: exp2(m_s - M)
+    __shared__ float linv;
+    const int t = blockIdx.x, h = blockIdx.y, c = threadIdx.x;
     const float* rec = part + ((size_t)t * H + h) * n_splits * ROW;
-    float M = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) M = fmaxf(M, rec[(size_t)s * ROW + HD]);
-    float L = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-        const float ms = rec[(size_t)s * ROW + HD];
-        L += (ms == -INFINITY) ? 0.f : exp2f(ms - M) * rec[(size_t)s * ROW + HD + 1];
-    }
-    const float inv = 1.0f / fmaxf(L, 1e-30f);
-    for (int c = threadIdx.x; c < HD; c += blockDim.x) {
-        float acc = 0.f;
-        for (int s = 0; s < n_splits; ++s) {
-            const float ms = rec[(size_t)s * ROW + HD];
-            if (ms != -INFINITY) acc += exp2f(ms - M) * rec[(size_t)s * ROW + c];
+    // the first wave turns the splits' maxima and sums into weights (up to 256 splits, 4 a lane)
+    if (c < 64) {
+        float ms[4], ls[4];
+        float M = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int s = c + u * 64;
+            ms[u] = s < n_splits ? rec[(size_t)s * ROW + HD] : -INFINITY;
+            ls[u] = s < n_splits ? rec[(size_t)s * ROW + HD + 1] : 0.f;
+            M = fmaxf(M, ms[u]);
         }
-        out[((size_t)t * H + h) * HD + c] = (bf16)(acc * inv);
+        M = wave_max(M);
+        float L = 0.f;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int s = c + u * 64;
+            const float w = (ms[u] == -INFINITY) ? 0.f : exp2f(ms[u] - M);
+            if (s < n_splits) wsh[s] = w;
+            L += w * ls[u];
+        }
+        L = wave_sum(L);
+        if (c == 0) linv = 1.0f / fmaxf(L, 1e-30f);
     }
+    __syncthreads();
+    float acc = 0.f;
+#pragma unroll 8
+    for (int s = 0; s < n_splits; ++s) acc += wsh[s] * rec[(size_t)s * ROW + c];
+    out[((size_t)t * H + h) * HD + c] = (bf16)(acc * linv);
 }
 
 // Bytes of fp32 scratch that a call needs.
@@ -182,7 +196,7 @@ extern "C" int spite_attn_decode(const void* q, const void* k_pages, const void*
     SP_REQUIRE(H / G <= 16, "attn_decode: %d query heads per kv head, at most 16", H / G);
     SP_REQUIRE(hd == 64 || hd == 128, "attn_decode: head size %d (this kernel has 64 and 128)", hd);
     SP_REQUIRE(page_size > 0 && page_size % 32 == 0, "attn_decode: page size %d must be a multiple of 32", page_size);
-    SP_REQUIRE(max_blocks > 0 && n_splits >= 1 && n_splits <= 65535, "attn_decode: bad table width or split count");
+    SP_REQUIRE(max_blocks > 0 && n_splits >= 1 && n_splits <= 256, "attn_decode: bad table width, or %d splits (at most 256)", n_splits);
     SP_REQUIRE(vis == SP_VIS_FULL || span > 0, "attn_decode: chunk or window of %d", span);
     SP_REQUIRE(G <= 65535 && T <= 65535, "attn_decode: too many heads or tokens for one launch");
     if (T == 0) return 0;
@@ -193,7 +207,7 @@ extern "C" int spite_attn_decode(const void* q, const void* k_pages, const void*
         attn_decode_kernel<128><<<grid, 256, sh, st>>>((const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages,
             (float*)workspace, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, n_splits);
         SP_LAUNCH_CHECK("attn_decode");
-        attn_decode_combine_kernel<128><<<dim3(T, H), 64, 0, st>>>((const float*)workspace, (bf16*)out, H, n_splits);
+        attn_decode_combine_kernel<128><<<dim3(T, H), 128, 0, st>>>((const float*)workspace, (bf16*)out, H, n_splits);
     } else {
         attn_decode_kernel<64><<<grid, 256, sh, st>>>((const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages,
             (float*)workspace, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, n_splits);

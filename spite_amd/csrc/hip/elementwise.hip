@@ -240,7 +240,7 @@ extern "C" int spite_rope_kvwrite(const void* qkv, void* q_out, void* k_pages, v
 // index wins a tie, weight = 1/(1+exp(-logit)).  The token's row sits in LDS; the waves take
 // the experts in turn, a lane's loads are independent 16-byte reads.  A logit's sum runs in
 // an order that depends on the width alone.
-#define ROUTER_NT 256
+#define ROUTER_NT 1024
 __global__ __launch_bounds__(ROUTER_NT)
 void router_top1_kernel(const float* __restrict__ x, const float* __restrict__ wr,
                         int* __restrict__ expert, float* __restrict__ weight,
@@ -258,7 +258,8 @@ void router_top1_kernel(const float* __restrict__ x, const float* __restrict__ w
         float acc = 0.f;
         if (vec) {
             const int nv = d >> 2;
-            for (int c = lane; c < nv; c += 64) {
+#pragma unroll 8
+            for (int c = lane; c < nv; c += 64) {          // independent 16-byte loads, several in flight
                 const f32x4 ww = ((const f32x4*)w)[c];
                 const f32x4 xx = ((const f32x4*)xs)[c];
                 acc += ww[0] * xx[0] + ww[1] * xx[1] + ww[2] * xx[2] + ww[3] * xx[3];

@@ -73,6 +73,62 @@ void sample_rows_kernel(const float* __restrict__ logits, int ld, int V, const f
     if (tid == 0) out[r] = found != 0x7fffffff ? found : bi;
 }
 
+// Arg-max in two stages when no row draws: the row is cut into slices, a workgroup finds the
+// best of its slice, a second kernel the best of the slices (lowest index among equals).
+#define ARG_SLICES 32
+__global__ __launch_bounds__(256)
+void argmax_slices_kernel(const float* __restrict__ logits, int ld, int V, float* __restrict__ pv, int* __restrict__ pi) {
+    __shared__ float sv[4];
+    __shared__ int si[4];
+    const int r = blockIdx.y, sl = blockIdx.x, tid = threadIdx.x;
+    const int per = (V + ARG_SLICES - 1) / ARG_SLICES;
+    const int b = sl * per, e = (b + per < V) ? b + per : V;
+    const float* row = logits + (size_t)r * ld;
+    float bv = 0.f; int bi = -1;
+#pragma unroll 4
+    for (int i = b + tid; i < e; i += 256) {
+        const float x = row[i];
+        if (bi < 0 || x > bv) { bv = x; bi = i; }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(bv, o, 64);
+        const int oi = __shfl_xor(bi, o, 64);
+        argmax_combine(bv, bi, ov, oi);
+    }
+    if ((tid & 63) == 0) { sv[tid >> 6] = bv; si[tid >> 6] = bi; }
+    __syncthreads();
+    if (tid == 0) {
+        for (int k = 1; k < 4; ++k) argmax_combine(bv, bi, sv[k], si[k]);
+        pv[r * ARG_SLICES + sl] = bv; pi[r * ARG_SLICES + sl] = bi;
+    }
+}
+__global__ void argmax_final_kernel(const float* __restrict__ pv, const int* __restrict__ pi, int* __restrict__ out) {
+    const int r = blockIdx.x;
+    float bv = pv[r * ARG_SLICES + threadIdx.x]; int bi = pi[r * ARG_SLICES + threadIdx.x];
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(bv, o, 64);
+        const int oi = __shfl_xor(bi, o, 64);
+        argmax_combine(bv, bi, ov, oi);
+    }
+    if (threadIdx.x == 0) out[r] = bi;
+}
+
+// `scratch`: n_rows * 32 floats and as many ints, for the two-stage arg-max (may be null:
+// then one workgroup walks each row).
+extern "C" int spite_argmax_rows(const float* logits, int ld, int n_rows, int V, float* scratch_v, int* scratch_i,
+                                 int* out, hipStream_t st) {
+    SP_REQUIRE(n_rows >= 0 && V > 0 && ld >= V, "argmax: bad sizes rows=%d V=%d ld=%d", n_rows, V, ld);
+    SP_REQUIRE(n_rows <= 65535, "argmax: too many rows");
+    if (n_rows == 0) return 0;
+    argmax_slices_kernel<<<dim3(ARG_SLICES, n_rows), 256, 0, st>>>(logits, ld, V, scratch_v, scratch_i);
+    SP_LAUNCH_CHECK("argmax_slices");
+    argmax_final_kernel<<<n_rows, ARG_SLICES, 0, st>>>(scratch_v, scratch_i, out);
+    SP_LAUNCH_CHECK("argmax_final");
+    return 0;
+}
+
 extern "C" int spite_sample_rows(const float* logits, int ld, int n_rows, int V, const float* temperature,
                                  const float* uniform, int* out, hipStream_t st) {
     SP_REQUIRE(n_rows >= 0 && V > 0 && ld >= V, "sample: bad sizes rows=%d V=%d ld=%d", n_rows, V, ld);

@@ -45,6 +45,7 @@ def lib():
             "spite_attn_decode": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, P],
             "spite_gemm_mfma": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, P],
             "spite_attn_prefill": [P, P, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, F, P],
+            "spite_argmax_rows": [P, I, I, I, P, P, P, P],
         }
         for name, args in sigs.items():
             fn = getattr(l, name)
@@ -339,3 +340,14 @@ def attn_prefill(q, k_pages, v_pages, out, positions, seq_of_token, cu_seqlens, 
         _ptr(cu_seqlens, "cu_seqlens", torch.int32), _ptr(block_table, "block_table", torch.int32),
         block_table.shape[1], _ptr(tile_start, "tile_start", torch.int32), int(n_tiles), H, G, hd, page_size,
         VIS[vis], int(span or 0), float(scale), _stream()), "attn_prefill")
+
+
+def argmax_rows(logits, out, scratch_v, scratch_i, n_rows=None):
+    """out[r] = index of the largest logit of row r, the lowest among equals.  Scratch: 32 floats
+    and 32 ints per row."""
+    n = n_rows if n_rows is not None else logits.shape[0]
+    if out.numel() < n or logits.shape[0] < n or scratch_v.numel() < 32 * n or scratch_i.numel() < 32 * n:
+        raise KernelError("argmax: outputs or scratch too small")
+    _check(lib().spite_argmax_rows(_ptr(logits, "logits", torch.float32), logits.stride(0), n, logits.shape[1],
+                                   _ptr(scratch_v, "scratch_v", torch.float32), _ptr(scratch_i, "scratch_i", torch.int32),
+                                   _ptr(out, "out", torch.int32), _stream()), "argmax")

@@ -83,7 +83,7 @@ class Attention(Mixer):
             if self.visibility != "full":
                 longest = min(longest, self.span + 32)
             blocks = -(-longest // 32)
-            n_splits = max(1, min(-(-1024 // (T * G)), -(-blocks // 4)))
+            n_splits = max(1, min(-(-1024 // (T * G)), -(-blocks // 4), 256))
             scratch = ws.take((hipops.attn_decode_workspace(T, H, hd, n_splits) // 4,), torch.float32)
             hipops.attn_decode(q, cache.k_pages, cache.v_pages, o, scratch, ctx.positions, ctx.seq_of_token,
                                cache.block_table, T, H, G, hd, cache.page_size, self.visibility, self.span,

@@ -45,6 +45,7 @@ class SamplingParams:
 class Sampler:
     def __init__(self, device):
         self.device = device
+        self._scratch = None
 
     def _process_row(self, row: torch.Tensor, p: SamplingParams, context: Sequence[int]) -> torch.Tensor:
         l = row.clone()
@@ -94,7 +95,10 @@ class Sampler:
                 rng_states[i], us[i] = lcg_next(rng_states[i])
         out = torch.empty(n, dtype=torch.int32, device=logits.device)
         if temps.max() <= 0:
-            hipops.sample_rows(work, None, None, out, n)
+            if self._scratch is None or self._scratch[0].numel() < 32 * n:
+                self._scratch = (torch.empty(32 * max(n, 64), dtype=torch.float32, device=logits.device),
+                                 torch.empty(32 * max(n, 64), dtype=torch.int32, device=logits.device))
+            hipops.argmax_rows(work, out, self._scratch[0], self._scratch[1], n)
         else:
             both = torch.from_numpy(np.stack([temps, us])).to(logits.device)
             hipops.sample_rows(work, both[0], both[1], out, n)
