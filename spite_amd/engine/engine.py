@@ -142,6 +142,15 @@ class Engine:
             ckpt_dtype = _CKPT_DTYPES.get(getattr(self.config, "torch_dtype", "bfloat16"), torch.bfloat16)
         self.spec = spec
         self.model = Model(spec, self.env)
+        self.page_size, self.max_batch_tokens, self.max_requests = int(page_size), int(max_batch_tokens), int(max_requests)
+        # the cache first, in one piece per group, then the weights: the loaders' temporaries
+        # (transposes, concatenations) must not cut the free memory into pieces before the
+        # large pools are taken
+        needs = self.model.cache_needs()
+        if num_pages is None:
+            tokens = cache_tokens if cache_tokens is not None else self.max_requests * 4096
+            num_pages = max(1, -(-int(tokens) // self.page_size))
+        self.cache = PagedCache(needs, self.page_size, num_pages, self.max_requests, self.env.dtype, self.device)
         if tensors is not None:
             self._load_from_dict(tensors, ckpt_dtype)
         elif random_weights:
@@ -150,12 +159,7 @@ class Engine:
             if not isinstance(model, str) or not os.path.isdir(model):
                 raise EngineError("without random_weights the model must be a folder with model.safetensors")
             load_weights(self.model, model, ckpt_dtype)
-        self.page_size, self.max_batch_tokens, self.max_requests = int(page_size), int(max_batch_tokens), int(max_requests)
-        needs = self.model.cache_needs()
-        if num_pages is None:
-            tokens = cache_tokens if cache_tokens is not None else self.max_requests * 4096
-            num_pages = max(1, -(-int(tokens) // self.page_size))
-        self.cache = PagedCache(needs, self.page_size, num_pages, self.max_requests, self.env.dtype, self.device)
+        torch.cuda.empty_cache()
         self._arenas = [Workspace(self.device), Workspace(self.device)]
         self._step_ws = Workspace(self.device)
         self._pin = None
