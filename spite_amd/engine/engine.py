@@ -166,7 +166,7 @@ class Engine:
         self._pin_event = None
         self._meta_dev = None
         self.steps_run = 0
-        self.use_graphs = bool(graphs)
+        self.use_graphs = bool(graphs) and self.model.graph_safe
         self._graphs: Dict[tuple, object] = {}     # shape of a decode step -> (graph, logits) or "seen"
         self._graph_stamp = None
         self.graph_replays = 0

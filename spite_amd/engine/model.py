@@ -33,6 +33,7 @@ class Model:
             if not call.write and (call.cache not in writers or writers[call.cache] > i):
                 raise ValueError(f"layer call {i} reads cache {call.cache} before any call has written it")
         self._writers = writers
+        self.graph_safe = all(b.graph_safe for b in self.blocks) and self.final_norm.graph_safe
 
     # ------------------------------------------------------------------ tensors
     def tensor_plan(self) -> List[Tuple[str, ParamSpec, object, str]]:

@@ -21,6 +21,8 @@ from ..csrc import hipops
 
 @register("mixer", "attention")
 class Attention(Mixer):
+    graph_safe = True
+
     def __init__(self, env, hidden_size, n_heads, n_kv_heads, head_dim, position, visibility="full", span=0,
                  qk_norm=False, qk_norm_eps=1e-5, temperature=None, softmax_scale=None):
         if n_heads % n_kv_heads:
@@ -36,6 +38,7 @@ class Attention(Mixer):
         self.temperature = temperature            # None or (floor_scale, attn_scale)
         self.scale = float(softmax_scale) if softmax_scale is not None else 1.0 / math.sqrt(self.hd)
         self.position = build_part("position", position, env)
+        self.graph_safe = self.position.graph_safe
         self.wqkv = self.wo = None
 
     def params(self):

@@ -87,6 +87,11 @@ class ModelSpec:
 class Part:
     """Base of all parts: declares its tensors and takes them when they are loaded."""
 
+    #: True when ``forward`` only launches work on the GPU whose arguments are the step's
+    #: device buffers: such a step can be captured in a graph and replayed.  A part that
+    #: reads the step's metadata on the host (``ctx.host``) must leave this False.
+    graph_safe = False
+
     def params(self) -> Dict[str, ParamSpec]:
         return {}
 

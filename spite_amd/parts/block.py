@@ -11,6 +11,8 @@ from .base import Block, register, build as build_part
 
 @register("block", "prenorm")
 class PreNormBlock(Block):
+    graph_safe = True
+
     def __init__(self, env, spec):
         self.env = env
         self.norm1 = build_part("norm", spec.norm1, env)
@@ -19,6 +21,7 @@ class PreNormBlock(Block):
         self.ffn = build_part("ffn", spec.ffn, env)
         self.children = (("norm1", self.norm1, spec.norm1), ("mixer", self.mixer, spec.mixer),
                          ("norm2", self.norm2, spec.norm2), ("ffn", self.ffn, spec.ffn))
+        self.graph_safe = all(part.graph_safe for _, part, _ in self.children)
 
     def forward(self, h, pending, ctx, cache):
         T, d = h.shape

@@ -20,6 +20,8 @@ from ..csrc import hipops
 
 @register("ffn", "dense_glu")
 class DenseGLU(FeedForward):
+    graph_safe = True
+
     def __init__(self, env, hidden_size, intermediate_size):
         self.d, self.F = int(hidden_size), int(intermediate_size)
         self.w_gate_up = self.w_down = None
@@ -44,6 +46,8 @@ class DenseGLU(FeedForward):
 
 @register("ffn", "moe_top1_sigmoid")
 class MoeTop1Sigmoid(FeedForward):
+    graph_safe = True
+
     wants_f32_input = True
 
     def __init__(self, env, hidden_size, intermediate_size, n_experts, shared_intermediate_size=None):

@@ -8,6 +8,8 @@ from ..csrc import hipops
 
 @register("norm", "rms")
 class RMSNorm(Norm):
+    graph_safe = True
+
     def __init__(self, env, width: int, eps: float):
         self.width = int(width)
         self.eps = float(eps)

@@ -41,6 +41,8 @@ def inv_frequencies(head_dim: int, theta: float, scaling=None):
 
 @register("position", "rotary")
 class Rotary(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, env, head_dim: int, theta: float, scaling=None, pairing: str = "half"):
         if head_dim % 2:
             raise ValueError(f"rotary: head size {head_dim} must be even")
@@ -58,5 +60,7 @@ class Rotary(PositionEncoding):
 
 @register("position", "none")
 class NoPosition(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, env):
         pass

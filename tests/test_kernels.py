@@ -371,3 +371,80 @@ def test_attention_refuses_what_it_cannot_do(kind):
             ops().attn_decode(z(1, 4 * 48), z(1, 2, 32, 48), z(1, 2, 48, 32), z(1, 4 * 48),
                               torch.zeros(4096, device=DEV), i32(1), i32(1), i32(1, 4), 1, 4, 2, 48, 32, "full", 0,
                               0.1, 1)                                    # head size 48
+
+
+# ------------------------------------------------------------------ router, expert plan, sampling
+@pytest.mark.parametrize("T,d,E", [(1, 64, 4), (9, 96, 8), (70, 5120, 16), (33, 1000, 128)])
+def test_router_and_plan(T, d, E):
+    x = rnd(T, d)
+    wr = rnd(E, d, seed=2)
+    wr[3 % E] = wr[1 % E]                                   # two experts with equal logits: the lower index wins
+    expert = torch.empty(T, dtype=torch.int32, device=DEV)
+    weight = torch.empty(T, dtype=torch.float32, device=DEV)
+    logits = torch.empty(T, E, dtype=torch.float32, device=DEV)
+    ops().router_top1(x, wr, expert, weight, logits)
+    idx, w, lg = plain.router_top1(x.double().cpu(), wr.double().cpu())
+    assert (logits.double().cpu() - lg).abs().max() < 2e-5 * lg.abs().max()
+    # where the plain side's two best logits are not within rounding of each other, the choice is the same
+    top2 = torch.topk(lg, 2, dim=-1).values
+    sure = (top2[:, 0] - top2[:, 1]) > 1e-4 * lg.abs().max()
+    assert torch.equal(expert.cpu().long()[sure], idx[sure])
+    assert not (expert.cpu() == 3 % E).any() or E <= 3      # the duplicate with the higher index is never taken
+    if sure.any():
+        assert (weight.double().cpu()[sure] - w[sure]).abs().max() < 1e-5
+    n = 2 * T
+    src, dst = torch.empty(n, dtype=torch.int32, device=DEV), torch.empty(n, dtype=torch.int32, device=DEV)
+    scale = torch.empty(n, dtype=torch.float32, device=DEV)
+    offsets = torch.empty(E + 2, dtype=torch.int32, device=DEV)
+    ops().moe_plan(expert, weight, src, scale, dst, offsets, T, E, True)
+    e, off, s_, d_ = expert.cpu().tolist(), offsets.cpu().tolist(), src.cpu().tolist(), dst.cpu().tolist()
+    assert off[0] == 0 and off[E] == T and off[E + 1] == 2 * T
+    for g in range(E):
+        members = s_[off[g]:off[g + 1]]
+        assert members == [t for t in range(T) if e[t] == g]        # stable: tokens in order inside a group
+    assert s_[T:] == list(range(T)) and d_[:T] == s_[:T] and d_[T:] == list(range(T, 2 * T))
+    assert torch.equal(scale[:T].cpu(), weight.cpu()[torch.tensor(s_[:T])]) and (scale[T:] == 1).all()
+
+
+@pytest.mark.parametrize("V", [7, 384, 202048])
+def test_argmax_and_sampling_rows(V):
+    from spite_amd.sampling.sampler import lcg_next
+    n = 5
+    logits = rnd(n, V, scale=3.0)
+    logits[0, V // 2] = logits[0].max() + 1
+    logits[1, 1] = logits[1, V - 2] = logits[1].max() + 2                  # a tie: the first wins
+    out = torch.empty(n, dtype=torch.int32, device=DEV)
+    sv, si = torch.empty(32 * n, device=DEV), torch.empty(32 * n, dtype=torch.int32, device=DEV)
+    ops().argmax_rows(logits, out, sv, si)
+    want = [plain.greedy(r) for r in logits.cpu()]
+    assert out.cpu().tolist() == want and want[0] == V // 2 and want[1] == 1
+    ops().sample_rows(logits, None, None, out)
+    assert out.cpu().tolist() == want
+    # draws: the same uniform numbers as the plain sampler's generator gives
+    temps = torch.tensor([0.0, 0.7, 1.0, 1.3, 2.0], device=DEV)
+    states, us, plain_tokens = [11, 12, 13, 14, 15], [], []
+    for r in range(n):
+        if float(temps[r]) > 0:
+            t, _ = plain.multinomial(logits[r].cpu() / float(temps[r]), states[r])
+            _, u = lcg_next(states[r])
+        else:
+            t, u = want[r], 0.0
+        plain_tokens.append(t)
+        us.append(u)
+    ops().sample_rows(logits, temps, torch.tensor(us, device=DEV), out)
+    got = out.cpu().tolist()
+    for r in range(n):
+        if got[r] != plain_tokens[r]:
+            # Both walk a float32 running sum over V terms, in different groupings; the sums
+            # differ by about sqrt(V) * 2^-24 of the total, so the two indices may lie apart
+            # by that much probability mass (and both must sit at the drawn number)
+            p = torch.softmax(logits[r].double().cpu() / float(temps[r]), 0)
+            cdf = torch.cumsum(p, 0)
+            slack = 4 * math.sqrt(V) * 2.0 ** -24 + 1e-6
+            assert abs(float(cdf[got[r]] - cdf[plain_tokens[r]])) < slack, (r, got[r], plain_tokens[r])
+            assert abs(float(cdf[got[r]]) - us[r]) < slack + float(p[got[r]])
+    # rows that were filtered to -inf are never drawn
+    masked = logits.clone()
+    masked[:, 1:] = float("-inf")
+    ops().sample_rows(masked, torch.ones(n, device=DEV), torch.rand(n, device=DEV), out)
+    assert out.cpu().tolist() == [0] * n
