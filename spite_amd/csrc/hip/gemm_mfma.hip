@@ -21,8 +21,8 @@
 #define MBK 64
 #define MLD (MBK + 8)      // padded row of the X tile in LDS, in elements
 
-template <int NW, bool GLU, typename TY>
-__global__ __launch_bounds__(NW * 64)
+template <int NW, bool GLU, bool EXACT, typename TY>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void gemm_mfma_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restrict__ W, long w_group_stride,
                       TY* __restrict__ Y, int ldy, int M, int N, int K,
                       const int* __restrict__ offsets, int n_groups, const int* __restrict__ a_rows,
@@ -80,33 +80,24 @@ void gemm_mfma_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restric
     }
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
     bf16x8 xr[XL];
-    bf16x8 w0[TA][2], w1[TA][2];   // two sets of W operands: [row tile][32-wide k step]
-    // `tail`: the tile runs past K (K is a multiple of 8, not of 64): chunks beyond it are zero
-    auto load_x = [&](int k0, bool tail) {
+    bf16x8 w0[TA][2], w1[TA][2];     // W operands of the even and of the odd tiles: [row tile][32-wide k step]
+    // EXACT: K is a multiple of the tile, no load carries a condition.  Otherwise chunks past
+    // K are zero (K is a multiple of 8); that form is slower and only serves odd widths.
+    auto load_x = [&](int k0) {
         const int k = k0 + lchunk * 8;
-        if (!tail) {
 #pragma unroll
-            for (int i = 0; i < XL; ++i) xr[i] = *(const bf16x8*)(xsrc[i] + k);
-        } else {
-#pragma unroll
-            for (int i = 0; i < XL; ++i) xr[i] = k < K ? *(const bf16x8*)(xsrc[i] + k) : zero;
-        }
+        for (int i = 0; i < XL; ++i) xr[i] = (EXACT || k < K) ? *(const bf16x8*)(xsrc[i] + k) : zero;
     };
     auto store_x = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < XL; ++i) *(bf16x8*)(Xs[buf] + (lrow + XR * i) * MLD + lchunk * 8) = xr[i];
     };
-    auto load_w = [&](bf16x8 (&w)[TA][2], int k0, bool tail) {
+    auto load_w = [&](bf16x8 (&ws)[TA][2], int k0) {
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
             const int k = k0 + kk * 32 + q * 8;
-            if (!tail) {
 #pragma unroll
-                for (int a = 0; a < TA; ++a) w[a][kk] = *(const bf16x8*)(wsrc[a] + k);
-            } else {
-#pragma unroll
-                for (int a = 0; a < TA; ++a) w[a][kk] = k < K ? *(const bf16x8*)(wsrc[a] + k) : zero;
-            }
+            for (int a = 0; a < TA; ++a) ws[a][kk] = (EXACT || k < K) ? *(const bf16x8*)(wsrc[a] + k) : zero;
         }
     };
 
@@ -115,7 +106,8 @@ void gemm_mfma_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restric
     for (int a = 0; a < TA; ++a)
 #pragma unroll
         for (int b = 0; b < 8; ++b) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
-    auto mul = [&](bf16x8 (&w)[TA][2], int buf) {
+    auto mul = [&](bf16x8 (&ws)[TA][2], int buf) {
+        const bf16* xs = Xs[buf];
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
 #pragma unroll
@@ -123,33 +115,46 @@ void gemm_mfma_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restric
                 bf16x8 xf[4];
 #pragma unroll
                 for (int b = 0; b < 4; ++b)
-                    xf[b] = *(const bf16x8*)(Xs[buf] + ((half * 4 + b) * 16 + r) * MLD + kk * 32 + q * 8);
+                    xf[b] = *(const bf16x8*)(xs + ((half * 4 + b) * 16 + r) * MLD + kk * 32 + q * 8);
 #pragma unroll
                 for (int a = 0; a < TA; ++a)
 #pragma unroll
                     for (int b = 0; b < 4; ++b)
-                        acc[a][half * 4 + b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[a][kk], xf[b], acc[a][half * 4 + b], 0, 0, 0);
+                        acc[a][half * 4 + b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ws[a][kk], xf[b], acc[a][half * 4 + b], 0, 0, 0);
             }
         }
     };
 
-    // tile t lives in Xs[t & 1] and in w0 (t even) or w1 (t odd)
-    auto is_tail = [&](int k0) { return k0 + MBK > K; };
-    load_x(0, is_tail(0));
-    load_w(w0, 0, is_tail(0));
+    // Tile t is multiplied out of Xs[t & 1] and w0 (t even) or w1 (t odd) while tile t+1 is
+    // in flight: its X chunks into registers (stored to the other LDS buffer after the
+    // products), its W operands into the other register set.
+    const int nt = (K + MBK - 1) / MBK;
+    load_x(0);
+    load_w(w0, 0);
     store_x(0);
     __syncthreads();
-    for (int k0 = 0; k0 < K; k0 += 2 * MBK) {
-        const bool more1 = k0 + MBK < K, more2 = k0 + 2 * MBK < K;
-        if (more1) { load_x(k0 + MBK, is_tail(k0 + MBK)); load_w(w1, k0 + MBK, is_tail(k0 + MBK)); }
+    int t = 0;
+    for (; t + 2 < nt; t += 2) {                 // steady state: no condition inside
+        load_x((t + 1) * MBK); load_w(w1, (t + 1) * MBK);
+        __builtin_amdgcn_sched_barrier(0);
         mul(w0, 0);
-        if (more1) store_x(1);
+        store_x(1);
         __syncthreads();
-        if (!more1) break;
-        if (more2) { load_x(k0 + 2 * MBK, is_tail(k0 + 2 * MBK)); load_w(w0, k0 + 2 * MBK, is_tail(k0 + 2 * MBK)); }
+        load_x((t + 2) * MBK); load_w(w0, (t + 2) * MBK);
+        __builtin_amdgcn_sched_barrier(0);
         mul(w1, 1);
-        if (more2) store_x(0);
+        store_x(0);
         __syncthreads();
+    }
+    if (t + 1 < nt) {                            // two tiles left
+        load_x((t + 1) * MBK); load_w(w1, (t + 1) * MBK);
+        __builtin_amdgcn_sched_barrier(0);
+        mul(w0, 0);
+        store_x(1);
+        __syncthreads();
+        mul(w1, 1);
+    } else {                                     // one tile left
+        mul(w0, 0);
     }
 
     // acc[a][b][i] of lane (r, q): column ncol[a] + q*4 + i, slot row0 + b*16 + r
@@ -197,8 +202,10 @@ extern "C" int spite_gemm_mfma(const void* X, int ldx, const void* W, long w_gro
     SP_REQUIRE(m_tiles <= 65535, "gemm_mfma: too many row tiles (%d)", m_tiles);
     const int ncols = glu ? MBN / 2 : MBN;
     dim3 grid((N + ncols - 1) / ncols, m_tiles);
-#define SP_MM(GLUV, TY) gemm_mfma_kernel<8, GLUV, TY><<<grid, 512, 0, st>>>((const bf16*)X, ldx, (const bf16*)W, \
-        w_group_stride, (TY*)Y, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows)
+#define SP_MM(GLUV, TY) do { if (K % MBK == 0) gemm_mfma_kernel<8, GLUV, true, TY><<<grid, 512, 0, st>>>((const bf16*)X, ldx, \
+        (const bf16*)W, w_group_stride, (TY*)Y, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows); \
+    else gemm_mfma_kernel<8, GLUV, false, TY><<<grid, 512, 0, st>>>((const bf16*)X, ldx, (const bf16*)W, \
+        w_group_stride, (TY*)Y, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows); } while (0)
     if (glu) { if (y_dtype == SP_BF16) SP_MM(true, bf16); else SP_MM(true, float); }
     else { if (y_dtype == SP_BF16) SP_MM(false, bf16); else SP_MM(false, float); }
 #undef SP_MM
