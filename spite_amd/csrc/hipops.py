@@ -10,6 +10,7 @@ from __future__ import annotations
 import ctypes
 from ctypes import c_int, c_long, c_float, c_void_p, c_size_t, c_char_p
 
+import numpy as np
 import torch
 
 from . import build
@@ -44,7 +45,7 @@ def lib():
             "spite_gemm_skinny": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, I, P],
             "spite_attn_decode": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, P],
             "spite_gemm_mfma": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, P],
-            "spite_attn_prefill": [P, P, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, F, P],
+            "spite_attn_prefill": [P, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, F, P],
             "spite_argmax_rows": [P, I, I, I, P, P, P, P],
         }
         for name, args in sigs.items():
@@ -318,28 +319,29 @@ def gemm_mfma(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_scal
         _stream()), "gemm_mfma")
 
 
-def attn_prefill(q, k_pages, v_pages, out, positions, seq_of_token, cu_seqlens, block_table, tile_start, n_tiles,
+def attn_prefill(q, k_pages, v_pages, out, positions, cu_seqlens, counts, block_table,
                  H, G, hd, page_size, vis, span, scale):
     """Prefill attention on MFMA (bf16; head sizes 64 and 128; pages of a multiple of 32 keys).
-    ``tile_start``: int32 row of q of the first query of every tile of at most 32 consecutive
-    queries of one request."""
+    ``counts``: the number of query tokens of every request of the step, on the host, in the
+    order of ``cu_seqlens`` (their running sum, on the device) and of the block table's rows."""
     if q.dtype != torch.bfloat16:
         raise KernelError(f"attn_prefill: bfloat16 only, got {q.dtype}")
-    T = positions.numel()
+    counts = np.ascontiguousarray(counts, dtype=np.int32)
+    n_seqs = int(counts.size)
+    T = int(counts.sum())
     if q.numel() < T * H * hd or out.numel() < T * H * hd:
         raise KernelError("attn_prefill: q or out too small")
     _check_pages(k_pages, v_pages, G, page_size, hd, "attn_prefill")
-    if block_table.dim() != 2 or seq_of_token.numel() < T or tile_start.numel() < n_tiles:
+    if block_table.dim() != 2 or block_table.shape[0] < n_seqs or positions.numel() < T:
         raise KernelError("attn_prefill: metadata too small")
-    if cu_seqlens.numel() < block_table.shape[0] + 1:
+    if cu_seqlens.numel() < n_seqs + 1:
         raise KernelError("attn_prefill: cu_seqlens shorter than the requests of the step")
     dt = torch.bfloat16
     _check(lib().spite_attn_prefill(
         _ptr(q, "q", dt), _ptr(k_pages, "k_pages", dt), _ptr(v_pages, "v_pages", dt), _ptr(out, "out", dt),
-        _ptr(positions, "positions", torch.int32), _ptr(seq_of_token, "seq_of_token", torch.int32),
-        _ptr(cu_seqlens, "cu_seqlens", torch.int32), _ptr(block_table, "block_table", torch.int32),
-        block_table.shape[1], _ptr(tile_start, "tile_start", torch.int32), int(n_tiles), H, G, hd, page_size,
-        VIS[vis], int(span or 0), float(scale), _stream()), "attn_prefill")
+        _ptr(positions, "positions", torch.int32), _ptr(cu_seqlens, "cu_seqlens", torch.int32),
+        counts.ctypes.data, n_seqs, _ptr(block_table, "block_table", torch.int32), block_table.shape[1],
+        H, G, hd, page_size, VIS[vis], int(span or 0), float(scale), _stream()), "attn_prefill")
 
 
 def argmax_rows(logits, out, scratch_v, scratch_i, n_rows=None):

@@ -93,8 +93,6 @@ class StepContext:
     n_out: int
     host: HostBatch
     ws: Any = None               # Workspace of the layer call that runs
-    qtile_start: Any = None      # int32 [n_qtiles]: first token row of every tile of <= 32 queries of one request
-    n_qtiles: int = 0
     decode_only: bool = False    # every entry holds one token
     max_count: int = 0           # longest portion of the step
     extras: dict = field(default_factory=dict)

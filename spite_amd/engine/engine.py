@@ -66,10 +66,9 @@ class StepMeta:
                     raise EngineError(f"entry {i}: wanted place {w} outside its {counts[i]} tokens")
                 rows.append(int(cu[i]) + int(w))
         n_out = len(rows)
-        qtiles = [int(cu[i]) + q0 for i in range(n) for q0 in range(0, int(counts[i]), 32)]
         # layout of the one int32 buffer
         sizes = [("token_ids", T), ("positions", T), ("seq_of_token", T), ("cu_seqlens", n + 1),
-                 ("seq_slots", n), ("seq_starts", n), ("logit_rows", n_out), ("qtile_start", len(qtiles))]
+                 ("seq_slots", n), ("seq_starts", n), ("logit_rows", n_out)]
         for g in range(n_groups):
             sizes += [(f"slot_map{g}", T), (f"table{g}", n * widths[g])]
         offs, total = {}, 0
@@ -87,7 +86,6 @@ class StepMeta:
         hv["seq_slots"][:] = slots
         hv["seq_starts"][:] = starts
         hv["logit_rows"][:] = np.asarray(rows, dtype=np.int32)
-        hv["qtile_start"][:] = np.asarray(qtiles, dtype=np.int32)
         for g in range(n_groups):
             cache.fill_step(slots, starts, counts, g, hv[f"slot_map{g}"], hv[f"table{g}"].reshape(n, widths[g]))
         dev = engine._upload(host, total)
@@ -97,7 +95,7 @@ class StepMeta:
         self.ctx = StepContext(
             T=T, n_seqs=n, token_ids=dv["token_ids"], positions=dv["positions"], seq_of_token=dv["seq_of_token"],
             cu_seqlens=dv["cu_seqlens"], seq_slots=dv["seq_slots"], seq_starts=dv["seq_starts"],
-            logit_rows=dv["logit_rows"], n_out=n_out, qtile_start=dv["qtile_start"], n_qtiles=len(qtiles),
+            logit_rows=dv["logit_rows"], n_out=n_out,
             host=HostBatch(slots=slots, starts=starts, counts=counts, cu_seqlens=cu),
             decode_only=bool(n > 0 and counts.max() == 1), max_count=int(counts.max()) if n else 0)
         self.host_tokens = tok[:T].copy()

@@ -92,9 +92,8 @@ class Attention(Mixer):
                                cache.block_table, T, H, G, hd, cache.page_size, self.visibility, self.span,
                                self.scale, n_splits)
         elif x.dtype == torch.bfloat16 and hd in (64, 128) and cache.page_size % 32 == 0:
-            hipops.attn_prefill(q, cache.k_pages, cache.v_pages, o, ctx.positions, ctx.seq_of_token, ctx.cu_seqlens,
-                                cache.block_table, ctx.qtile_start, ctx.n_qtiles, H, G, hd, cache.page_size,
-                                self.visibility, self.span, self.scale)
+            hipops.attn_prefill(q, cache.k_pages, cache.v_pages, o, ctx.positions, ctx.cu_seqlens, ctx.host.counts,
+                                cache.block_table, H, G, hd, cache.page_size, self.visibility, self.span, self.scale)
         else:
             hipops.attn_generic(q, cache.k_pages, cache.v_pages, o, ctx.positions, ctx.seq_of_token,
                                 cache.block_table, T, H, G, hd, cache.page_size, self.visibility, self.span,

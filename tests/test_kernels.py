@@ -256,6 +256,16 @@ def run_attention(kind, dtype, H, G, hd, ps, lens, queries, vis, span, n_splits=
     scale = 1.0 / math.sqrt(hd)
     if kind == "generic":
         ops().attn_generic(q_dev, kp, vp, out, positions, seq, bt, T, H, G, hd, ps, vis, span, scale)
+    elif kind == "prefill":                      # runs of queries of one request are the portions
+        runs = []
+        for s, _ in queries:
+            if runs and runs[-1][0] == s:
+                runs[-1][1] += 1
+            else:
+                runs.append([s, 1])
+        cu = torch.tensor([0] + list(np.cumsum([c for _, c in runs])), dtype=torch.int32, device=DEV)
+        ops().attn_prefill(q_dev, kp, vp, out, positions, cu, [c for _, c in runs],
+                           bt[[s for s, _ in runs]].contiguous(), H, G, hd, ps, vis, span, scale)
     else:
         wsz = ops().attn_decode_workspace(T, H, hd, n_splits)
         scratch = torch.empty(wsz // 4, dtype=torch.float32, device=DEV)
@@ -314,6 +324,10 @@ PORTION_CASES = [
     (40, 8, 128, 64, [130, 65], [(0, 97, 33), (1, 0, 65)], "full", 0),
     (16, 1, 64, 32, [500], [(0, 380, 120)], "window", 100),
     (12, 4, 128, 32, [260, 70], [(0, 258, 2), (1, 0, 70)], "chunk", 64),
+    (6, 2, 128, 64, [900], [(0, 0, 900)], "full", 0),                          # 3 heads a kv head: tiles of 85 queries
+    (2, 2, 64, 32, [600, 3], [(0, 100, 500), (1, 0, 3)], "full", 0),           # one head a kv head: tiles of 256
+    (40, 8, 128, 64, [700], [(0, 300, 400)], "window", 257),
+    (34, 2, 64, 96, [400], [(0, 0, 400)], "full", 0),                          # 17 heads a kv head, pages of 96
 ]
 
 
@@ -334,16 +348,24 @@ def test_attn_prefill(case):
     cu = [0]
     for _, _, count in portions:
         cu.append(cu[-1] + count)
-    tiles = [cu[i] + q0 for i, (_, _, count) in enumerate(portions) for q0 in range(0, count, 32)]
     bt = torch.stack([kv.bt[s] for s, _, _ in portions]).to(DEV)
     out = torch.zeros(T, H * hd, dtype=dtype, device=DEV)
-    ops().attn_prefill(qs.reshape(T, H * hd).to(DEV), kv.kp.to(DEV), kv.vp.to(DEV), out, positions, seq,
-                       torch.tensor(cu, dtype=torch.int32, device=DEV), bt,
-                       torch.tensor(tiles, dtype=torch.int32, device=DEV), len(tiles), H, G, hd, ps, vis, span,
-                       1.0 / math.sqrt(hd))
+    ops().attn_prefill(qs.reshape(T, H * hd).to(DEV), kv.kp.to(DEV), kv.vp.to(DEV), out, positions,
+                       torch.tensor(cu, dtype=torch.int32, device=DEV), [count for _, _, count in portions], bt,
+                       H, G, hd, ps, vis, span, 1.0 / math.sqrt(hd))
     got = out.double().cpu().view(T, H, hd)
     assert torch.isfinite(got).all()
     assert (got - ref).abs().max() < 1.5e-2 * max(1.0, float(ref.abs().max()))
+
+
+def test_prefill_attention_finds_one_far_key_among_thousands():
+    # as below, for one query in the middle of a portion of 100: the far key lies in a block
+    # that every query of the tile sees whole
+    queries = [(0, p) for p in range(2900, 3000)]
+    got, ref = run_attention("prefill", torch.bfloat16, 8, 2, 128, 64, [3000], queries, "full", 0, planted=(50, 0, 77))
+    kv = PagedKV([3000], 2, 128, 64, torch.bfloat16, 0)
+    assert (ref[50, 0] - kv.v[0][77][0].double()).abs().max() < 0.05
+    assert (got - ref).abs().max() < 2e-2
 
 
 @pytest.mark.parametrize("kind", ["generic", "decode"])
