@@ -81,6 +81,8 @@ def main() -> int:
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--tiny", action="store_true", help="a small model of the same kind, to try the script")
     ap.add_argument("--no-graphs", action="store_true", help="run decode steps eagerly (for kernel traces)")
+    ap.add_argument("--phase", default="all", choices=["all", "decode", "prefill"],
+                    help="time only one phase (for kernel traces); the other's figures are null")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not measured")
@@ -125,12 +127,18 @@ def main() -> int:
         dt = time.perf_counter() - t
         eng.release(s)
         return dt
-    prefill_once()
-    pre = min(prefill_once() for _ in range(2))
-    pf = prefill_flops(cfg, L, args.prefill_tokens)
-    prefill = {"value": round(args.prefill_tokens / pre, 1), "tokens": args.prefill_tokens,
-               "ms": round(pre * 1e3, 3), "frac": round(pf / pre / MFMA_PEAK[args.dtype], 4)}
-    log(f"prefill {args.prefill_tokens} tokens: {pre * 1e3:.1f} ms")
+    prefill = None
+    if args.phase != "decode":
+        prefill_once()
+        pre = min(prefill_once() for _ in range(2))
+        pf = prefill_flops(cfg, L, args.prefill_tokens)
+        prefill = {"value": round(args.prefill_tokens / pre, 1), "tokens": args.prefill_tokens,
+                   "ms": round(pre * 1e3, 3), "frac": round(pf / pre / MFMA_PEAK[args.dtype], 4)}
+        log(f"prefill {args.prefill_tokens} tokens: {pre * 1e3:.1f} ms")
+    if args.phase == "prefill":
+        print(json.dumps({"metric": "prefill only", "value": None, "prefill": prefill, "n_gpus": 1,
+                          "config": {"layers": L, "layers_full": layers_full}}))
+        return 0
 
     # ---- decode at a fixed batch
     def fill_context(slots):
