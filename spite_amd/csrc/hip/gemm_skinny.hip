@@ -15,10 +15,14 @@
 //    (W.(s x) = s (W.x)), so the scaled input is never rounded.  With GLU the workgroup also
 //    owns the matching "up" rows N+n and writes silu(gate) * up.
 //
+//  * TILED: W lies in MFMA operand order (see gemm_tiled.hip: tiles of 16 rows x 32 k, each
+//    one kilobyte in lane order).  A lane's loads are then the tile's 16 bytes at lane * 16,
+//    and k runs q*8 .. q*8+7 inside every 32: X is read to match.
+//
 // A row's sum runs over k in an order that does not depend on M or on the other rows.
 #include "common.h"
 
-template <int R, int G, int S, int NW, bool GLU, typename TY>
+template <int R, int G, int S, int NW, bool GLU, bool TILED, typename TY>
 __global__ __launch_bounds__(NW * 64)
 void gemm_skinny_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restrict__ W, long w_group_stride,
                         TY* __restrict__ Y, int ldy, int M, int N, int K,
@@ -60,7 +64,8 @@ void gemm_skinny_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restr
         int n = n0 + (a % R) * 16 + r;
         n = n < N ? n : N - 1;
         const size_t row = (GLU && a >= R) ? (size_t)N + n : (size_t)n;
-        wp[a] = Wg + row * K;
+        if (TILED) wp[a] = Wg + (row / 16) * (size_t)(K / 32) * 512 + lane * 8;     // the row's band; N % 16 == 0
+        else wp[a] = Wg + row * K;
     }
     const bf16* xp[G];
 #pragma unroll
@@ -83,9 +88,10 @@ void gemm_skinny_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restr
     auto load = [&](bf16x8 (&wa)[RA][S], bf16x8 (&xb)[G][S], int kb) {
 #pragma unroll
         for (int s = 0; s < S; ++s) {
-            const int k = kb + q * (8 * S) + s * 8;
+            const int k = TILED ? kb + s * 32 + q * 8 : kb + q * (8 * S) + s * 8;
+            const size_t kw = TILED ? (size_t)(kb / 32 + s) * 512 : (size_t)k;
 #pragma unroll
-            for (int a = 0; a < RA; ++a) wa[a][s] = *(const bf16x8*)(wp[a] + k);
+            for (int a = 0; a < RA; ++a) wa[a][s] = *(const bf16x8*)(wp[a] + kw);
 #pragma unroll
             for (int b = 0; b < G; ++b) xb[b][s] = *(const bf16x8*)(xp[b] + k);
         }
@@ -94,9 +100,10 @@ void gemm_skinny_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restr
     auto load_tail = [&](bf16x8 (&wa)[RA][S], bf16x8 (&xb)[G][S], int kb) {
 #pragma unroll
         for (int s = 0; s < S; ++s) {
-            const int k = kb + q * (8 * S) + s * 8;
+            const int k = TILED ? kb + s * 32 + q * 8 : kb + q * (8 * S) + s * 8;
+            const size_t kw = TILED ? (size_t)(kb / 32 + s) * 512 : (size_t)k;
 #pragma unroll
-            for (int a = 0; a < RA; ++a) wa[a][s] = k < K ? *(const bf16x8*)(wp[a] + k) : zero;
+            for (int a = 0; a < RA; ++a) wa[a][s] = k < K ? *(const bf16x8*)(wp[a] + kw) : zero;
 #pragma unroll
             for (int b = 0; b < G; ++b) xb[b][s] = k < K ? *(const bf16x8*)(xp[b] + k) : zero;
         }
@@ -161,14 +168,14 @@ void gemm_skinny_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restr
 template <int R, int G, int S, int NW>
 static int launch_skinny(const void* X, int ldx, const void* W, long wgs, void* Y, int y_dtype, int ldy, int M, int N,
                          int K, const int* offsets, int n_groups, const int* a_rows, const float* a_scale,
-                         const int* y_rows, int glu, hipStream_t st) {
+                         const int* y_rows, int glu, int tiled, hipStream_t st) {
     const int MT = 16 * G;
     const int m_tiles = (M + MT - 1) / MT + (offsets ? n_groups : 0);
     SP_REQUIRE(m_tiles <= 65535, "gemm_skinny: too many row tiles (%d)", m_tiles);
     dim3 grid((N + 16 * R - 1) / (16 * R), m_tiles);
     const size_t sh = (size_t)NW * (glu ? 2 : 1) * R * G * 4 * 64 * sizeof(float);
 #define SP_SK(GLUV, TY) do { \
-        auto kern = gemm_skinny_kernel<R, G, S, NW, GLUV, TY>; \
+        auto kern = tiled ? gemm_skinny_kernel<R, G, S, NW, GLUV, true, TY> : gemm_skinny_kernel<R, G, S, NW, GLUV, false, TY>; \
         if (sh > 48 * 1024) { hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sh); \
             if (e != hipSuccess) return sp_fail("gemm_skinny: cannot get %zu bytes of LDS: %s", sh, hipGetErrorString(e)); } \
         kern<<<grid, NW * 64, sh, st>>>((const bf16*)X, ldx, (const bf16*)W, wgs, (TY*)Y, ldy, M, N, K, offsets, \
@@ -185,14 +192,15 @@ static int launch_skinny(const void* X, int ldx, const void* W, long wgs, void* 
 extern "C" int spite_gemm_skinny(const void* X, int ldx, const void* W, long w_group_stride, void* Y, int y_dtype,
                                  int ldy, int M, int N, int K, const int* offsets, int n_groups, const int* a_rows,
                                  const float* a_scale, const int* y_rows, int glu, int max_rows, int variant,
-                                 hipStream_t st) {
+                                 int w_tiled, hipStream_t st) {
     SP_REQUIRE(M >= 0 && N > 0 && K > 0 && ldx >= K && ldy >= N, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
     SP_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "gemm_skinny: K=%d and the row stride %d must be multiples of 8", K, ldx);
     SP_REQUIRE(((uintptr_t)X & 15) == 0 && ((uintptr_t)W & 15) == 0, "gemm_skinny: operands must be 16-byte aligned");
     SP_REQUIRE(y_dtype == SP_BF16 || y_dtype == SP_F32, "gemm_skinny: output dtype %d", y_dtype);
     SP_REQUIRE(!offsets || n_groups > 0, "gemm_skinny: grouped call without groups");
+    SP_REQUIRE(!w_tiled || (K % 32 == 0 && N % 16 == 0), "gemm_skinny: operand order needs K=%d a multiple of 32 and N=%d of 16", K, N);
     if (M == 0) return 0;
-#define SP_ARGS X, ldx, W, w_group_stride, Y, y_dtype, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, st
+#define SP_ARGS X, ldx, W, w_group_stride, Y, y_dtype, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, w_tiled, st
     // measured on MI355X (GB/s of W at Llama 4 Scout's shapes): one row tile per workgroup for
     // the experts' grouped stream, two for the dense projections, four for the output matrix
     if (variant == 0) {

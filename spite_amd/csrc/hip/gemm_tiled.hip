@@ -1,0 +1,243 @@
+// Tiled bf16 product for many rows (prefill) over weights stored in MFMA operand order:
+// Y[M,N] = X[M,K] . W[N,K]^T, fp32 accumulation on MFMA 16x16x32.
+//
+// "Operand order" of W[N,K] (N % 16 == 0, K % 64 == 0): the matrix is cut into tiles of 16
+// rows x 32 k; tile (i, j) lies at ((i * K/32) + j) * 512 elements, and inside it the eight
+// elements W[16i + r][32j + 8q .. 8q+7] lie at ((q*16 + r) * 8): exactly what lane q*16 + r of
+// a wave holds as the MFMA "A" operand.  A wave's load of a tile is one kilobyte in a row,
+// eight whole cache lines, where the same load from a row-major matrix touches sixteen half
+// lines; the path from L2 into the registers carries about half again as much that way, and
+// that path, not the MFMA units or LDS, is what bounds this kernel.  The tiles of one row
+// band follow each other in k, so a wave streams its four bands.
+//
+// A workgroup of eight waves owns 128*WM rows of X ("slots") and 64*WN rows of W
+// (WN * WM = 8); a wave owns 64 rows of W and 128 slots: 4 x 8 accumulator tiles.
+//  * W never touches LDS: three rotating sets of operand registers, loaded two steps of 32 k
+//    ahead of the products.
+//  * X is the "B" operand, shared by the waves: tiles of 64 k go through LDS, fetched with
+//    eight lanes a row (whole cache lines), rows padded by 16 bytes against bank conflicts,
+//    double-buffered, one barrier per 64 k.
+//  * Tiles are handed out so that the workgroups running on one XCD (one L2) at a time share
+//    W bands and walk K together.
+// Grouped form (experts) and GLU as in gemm_generic.hip; with GLU a wave's bands are two of
+// gate rows and the two matching of up rows.
+#include "common.h"
+
+#define TLD 72             // padded row of the X tile in LDS, in elements (64 k + 8)
+
+template <int WN, int WM, bool GLU, typename TY>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restrict__ W, long w_group_stride,
+                       TY* __restrict__ Y, int ldy, int M, int N, int K,
+                       const int* __restrict__ offsets, int n_groups, const int* __restrict__ a_rows,
+                       const float* __restrict__ a_scale, const int* __restrict__ y_rows, int m_tiles, int n_tiles) {
+    static_assert(WN * WM == 8, "eight waves");
+    constexpr int BM = 128 * WM, BN = 64 * WN;
+    constexpr int NCOLS = GLU ? BN / 2 : BN;        // output columns per workgroup
+    extern __shared__ __attribute__((aligned(16))) bf16 Xs[];     // [2][BM * TLD]
+
+    // Which tile.  Workgroups go to the eight XCDs in turn, each with an L2 of its own: XCD x
+    // takes the x-th eighth of the tiles, ordered with the row tile running fastest.
+    const int per_xcd = (m_tiles * n_tiles + 7) / 8;
+    const int tile_id = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (tile_id >= m_tiles * n_tiles) return;
+    const int tile_m = tile_id % m_tiles, tile_n = tile_id / m_tiles;
+    int g = 0, row0, row_end = M;
+    if (offsets) {
+        int mt = tile_m, acc = 0;
+        g = -1;
+        for (int e = 0; e < n_groups; ++e) {
+            const int b = offsets[e], en = offsets[e + 1];
+            const int nt = (en - b + BM - 1) / BM;
+            if (mt < acc + nt) { g = e; row0 = b + (mt - acc) * BM; row_end = en; break; }
+            acc += nt;
+        }
+        if (g < 0) return;
+    } else {
+        row0 = tile_m * BM;
+        if (row0 >= M) return;
+    }
+    const int n0 = tile_n * NCOLS;
+    const bf16* Wg = W + (size_t)g * w_group_stride;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wn = wave % WN, wm = wave / WN;
+    const int r = lane & 15, q = lane >> 4;
+
+    // ---- X: global -> registers -> LDS; thread loads 16-byte chunk (tid % 8) of rows tid/8 + 64*i
+    constexpr int XL = 2 * WM;
+    const int lrow = tid >> 3, lchunk = tid & 7;
+    const bf16* xsrc[XL];
+#pragma unroll
+    for (int i = 0; i < XL; ++i) {
+        // rows past the group read its last row again: no load of the main loop carries a
+        // condition, and what such rows produce is never stored
+        int s = row0 + lrow + 64 * i;
+        s = s < row_end ? s : row_end - 1;
+        xsrc[i] = X + (size_t)(a_rows ? a_rows[s] : s) * ldx + lchunk * 8;
+    }
+    // ---- W: the wave's four row bands
+    //      plain: rows n0 + wn*64 + a*16; GLU: bands 0, 1 gate rows n0 + wn*32 + ..., bands 2, 3 the up rows N + ...
+    constexpr int TG = GLU ? 2 : 4;          // bands that name distinct output columns
+    const int kt = K / 32;                   // tiles in a band
+    const bf16* wsrc[4];
+    int ncol[4];                             // output column of the band's first row
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+        const int n = n0 + wn * 16 * TG + (a % TG) * 16;
+        int band = n / 16;
+        band = band < N / 16 ? band : N / 16 - 1;        // bands past N read the last band again
+        if (GLU && a >= TG) band += N / 16;
+        ncol[a] = n;
+        wsrc[a] = Wg + (size_t)band * kt * 512 + lane * 8;
+    }
+    const int nu = K / 64;
+    auto load_x = [&](bf16x8 (&xr)[XL], int u) {
+        const int k0 = (u < nu ? u : nu - 1) * 64;
+#pragma unroll
+        for (int i = 0; i < XL; ++i) xr[i] = *(const bf16x8*)(xsrc[i] + k0);
+    };
+    auto store_x = [&](bf16x8 (&xr)[XL], int buf) {
+#pragma unroll
+        for (int i = 0; i < XL; ++i) *(bf16x8*)(Xs + buf * (BM * TLD) + (lrow + 64 * i) * TLD + lchunk * 8) = xr[i];
+    };
+    auto load_w = [&](bf16x8 (&ws)[4], int t) {
+        const size_t at = (size_t)(t < kt ? t : kt - 1) * 512;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) ws[a] = *(const bf16x8*)(wsrc[a] + at);
+    };
+
+    f32x4 acc[4][8];           // [W band a][slot tile b]
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 8; ++b) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+    auto mul = [&](bf16x8 (&ws)[4], int buf, int kk) {
+        const bf16* xs = Xs + buf * (BM * TLD) + (wm * 128 + r) * TLD + kk * 32 + q * 8;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            bf16x8 xf[4];
+#pragma unroll
+            for (int b = 0; b < 4; ++b) xf[b] = *(const bf16x8*)(xs + (half * 4 + b) * 16 * TLD);
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+#pragma unroll
+                for (int b = 0; b < 4; ++b)
+                    acc[a][half * 4 + b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ws[a], xf[b], acc[a][half * 4 + b], 0, 0, 0);
+        }
+    };
+
+    // Step u covers 64 k: two half steps t = 2u, 2u+1.  Half step t multiplies W set t % 3
+    // with the X tile in LDS buffer u % 2 while W tile t+2 is asked for into set (t+2) % 3.
+    // X tile u+1 is asked for at the start of step u and stored to the other LDS buffer at
+    // its end.  Three steps bring every name back; the loop has one way out (leaving it from
+    // the middle made the compiler spill the accumulators), so its last round may run past
+    // the end: only its loads happen then, of the last tile again.
+    bf16x8 w0[4], w1[4], w2[4], xr[XL];
+    auto step = [&](bf16x8 (&wa)[4], bf16x8 (&wb)[4], bf16x8 (&wc)[4], int u) {
+        // wa: set of half step 2u, wb: of 2u+1, wc: of 2u+2
+        load_x(xr, u + 1);
+        load_w(wc, 2 * u + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        if (u < nu) mul(wa, u & 1, 0);
+        load_w(wa, 2 * u + 3);
+        __builtin_amdgcn_sched_barrier(0);
+        if (u < nu) mul(wb, u & 1, 1);
+        store_x(xr, (u + 1) & 1);
+        __syncthreads();
+    };
+    load_x(xr, 0);
+    load_w(w0, 0);
+    load_w(w1, 1);
+    store_x(xr, 0);
+    __syncthreads();
+    for (int u = 0; u < nu; u += 3) {
+        step(w0, w1, w2, u);            // half steps 0, 1: use w0, w1; load w2 (t=2), w0 (t=3)
+        step(w2, w0, w1, u + 1);        // half steps 2, 3: use w2, w0; load w1 (t=4), w2 (t=5)
+        step(w1, w2, w0, u + 2);        // half steps 4, 5: use w1, w2; load w0 (t=6), w1 (t=7)
+    }
+
+    // acc[a][b][i] of lane (r, q): column ncol[a] + q*4 + i, slot row0 + wm*128 + b*16 + r
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+        const int s = row0 + wm * 128 + b * 16 + r;
+        if (s >= row_end) continue;
+        const float sc = a_scale ? a_scale[s] : 1.0f;
+        const size_t yr = y_rows ? (size_t)y_rows[s] : (size_t)s;
+        TY* yrow = Y + yr * ldy;
+        if (GLU) {
+#pragma unroll
+            for (int a = 0; a < TG; ++a) {
+                const int n = ncol[a] + q * 4;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    if (n + i < N) {
+                        const float gv = acc[a][b][i] * sc, uv = acc[a + TG][b][i] * sc;
+                        yrow[n + i] = from_f32<TY>(gv / (1.0f + __expf(-gv)) * uv);
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                const int n = ncol[a] + q * 4;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (n + i < N) yrow[n + i] = from_f32<TY>(acc[a][b][i] * sc);
+            }
+        }
+    }
+}
+
+template <int WN, int WM, bool GLU, typename TY>
+static int launch_tiled_kernel(const void* X, int ldx, const void* W, long w_group_stride, void* Y, int ldy, int M, int N,
+                               int K, const int* offsets, int n_groups, const int* a_rows, const float* a_scale,
+                               const int* y_rows, hipStream_t st) {
+    constexpr int BM = 128 * WM, BN = 64 * WN;
+    const int m_tiles = (M + BM - 1) / BM + (offsets ? n_groups : 0);
+    const int ncols = GLU ? BN / 2 : BN;
+    const int n_tiles = (N + ncols - 1) / ncols;
+    SP_REQUIRE((long)m_tiles * n_tiles < (1L << 30), "gemm_tiled: too many tiles");
+    const size_t sh = (size_t)2 * BM * TLD * sizeof(bf16);
+    static bool allowed = false;        // one flag per instantiation; more LDS than the default limit for WM = 2
+    if (!allowed) {
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<WN, WM, GLU, TY>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)sh);
+        SP_REQUIRE(e == hipSuccess, "gemm_tiled: %zu bytes of LDS refused: %s", sh, hipGetErrorString(e));
+        allowed = true;
+    }
+    gemm_tiled_kernel<WN, WM, GLU, TY><<<dim3((m_tiles * n_tiles + 7) / 8 * 8), 512, sh, st>>>(
+        (const bf16*)X, ldx, (const bf16*)W, w_group_stride, (TY*)Y, ldy, M, N, K, offsets, n_groups, a_rows, a_scale,
+        y_rows, m_tiles, n_tiles);
+    SP_LAUNCH_CHECK("gemm_tiled");
+    return 0;
+}
+
+template <int WN, int WM>
+static int launch_tiled(const void* X, int ldx, const void* W, long w_group_stride, void* Y, int y_dtype, int ldy, int M,
+                        int N, int K, const int* offsets, int n_groups, const int* a_rows, const float* a_scale,
+                        const int* y_rows, int glu, hipStream_t st) {
+#define SP_TL(GLUV, TY) launch_tiled_kernel<WN, WM, GLUV, TY>(X, ldx, W, w_group_stride, Y, ldy, M, N, K, offsets, n_groups, \
+                                                              a_rows, a_scale, y_rows, st)
+    if (glu) return y_dtype == SP_BF16 ? SP_TL(true, bf16) : SP_TL(true, float);
+    return y_dtype == SP_BF16 ? SP_TL(false, bf16) : SP_TL(false, float);
+#undef SP_TL
+}
+
+// W in operand order (see above), every group N (2N with GLU) rows of K.
+// `shape`: 0 lets the library choose; 1 = 512 W rows x 128 slots a workgroup, 2 = 256 x 256.
+extern "C" int spite_gemm_tiled(const void* X, int ldx, const void* W, long w_group_stride, void* Y, int y_dtype,
+                                int ldy, int M, int N, int K, const int* offsets, int n_groups, const int* a_rows,
+                                const float* a_scale, const int* y_rows, int glu, int shape, hipStream_t st) {
+    SP_REQUIRE(M >= 0 && N > 0 && K > 0 && ldx >= K && ldy >= N, "gemm_tiled: bad sizes M=%d N=%d K=%d", M, N, K);
+    SP_REQUIRE(K % 64 == 0 && N % 16 == 0, "gemm_tiled: operand order needs K=%d a multiple of 64 and N=%d of 16", K, N);
+    SP_REQUIRE(ldx % 8 == 0, "gemm_tiled: the row stride %d must be a multiple of 8", ldx);
+    SP_REQUIRE(((uintptr_t)X & 15) == 0 && ((uintptr_t)W & 15) == 0, "gemm_tiled: operands must be 16-byte aligned");
+    SP_REQUIRE(y_dtype == SP_BF16 || y_dtype == SP_F32, "gemm_tiled: output dtype %d", y_dtype);
+    SP_REQUIRE(!offsets || n_groups > 0, "gemm_tiled: grouped call without groups");
+    SP_REQUIRE(shape >= 0 && shape <= 2, "gemm_tiled: tile shape %d", shape);
+    if (M == 0) return 0;
+    if (shape == 0) shape = (offsets || M <= 128) ? 1 : 2;
+    if (shape == 1)
+        return launch_tiled<8, 1>(X, ldx, W, w_group_stride, Y, y_dtype, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, st);
+    return launch_tiled<4, 2>(X, ldx, W, w_group_stride, Y, y_dtype, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, st);
+}

@@ -42,9 +42,10 @@ def lib():
             "spite_gemm_generic": [P, I, P, L, I, P, I, I, I, I, I, P, I, P, P, P, I, P],
             "spite_attn_generic": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, P],
             "spite_sample_rows": [P, I, I, I, P, P, P, P],
-            "spite_gemm_skinny": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, I, P],
+            "spite_gemm_skinny": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, I, I, P],
             "spite_attn_decode": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, P],
-            "spite_gemm_mfma": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, P],
+            "spite_gemm_mfma": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, P],
+            "spite_gemm_tiled": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, P],
             "spite_attn_prefill": [P, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, F, P],
             "spite_argmax_rows": [P, I, I, I, P, P, P, P],
         }
@@ -267,9 +268,10 @@ def _gemm_checks(a, w, y, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, g
 
 
 def gemm_skinny(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None,
-                glu=False, max_rows=None, variant=0):
+                glu=False, max_rows=None, variant=0, tiled=False):
     """Weight-streaming bf16 product for few rows (see gemm_skinny.hip); arguments as gemm_generic.
-    ``max_rows``: the most rows a group can bring (default M)."""
+    ``max_rows``: the most rows a group can bring (default M).  ``tiled``: w is in MFMA operand
+    order (``operand_order``)."""
     rows_w = _gemm_checks(a, w, y, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, "gemm_skinny")
     if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise KernelError(f"gemm_skinny: bfloat16 operands only, got {a.dtype} and {w.dtype}")
@@ -277,7 +279,7 @@ def gemm_skinny(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_sc
         _ptr(a, "a"), a.stride(0), _ptr(w, "w"), rows_w * K, _ptr(y, "y"), dtype_code(y.dtype), y.stride(0),
         M, N, K, _ptr(offsets, "offsets", torch.int32, True), n_groups, _ptr(a_rows, "a_rows", torch.int32, True),
         _ptr(a_scale, "a_scale", torch.float32, True), _ptr(y_rows, "y_rows", torch.int32, True), int(glu),
-        int(max_rows if max_rows is not None else M), int(variant), _stream()), "gemm_skinny")
+        int(max_rows if max_rows is not None else M), int(variant), int(bool(tiled)), _stream()), "gemm_skinny")
 
 
 def attn_decode_workspace(T, H, hd, n_splits) -> int:
@@ -307,7 +309,8 @@ def attn_decode(q, k_pages, v_pages, out, workspace, positions, seq_of_token, bl
         _stream()), "attn_decode")
 
 
-def gemm_mfma(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None, glu=False):
+def gemm_mfma(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None, glu=False,
+              shape=0):
     """Tiled bf16 MFMA product for many rows (see gemm_mfma.hip); arguments as gemm_generic."""
     rows_w = _gemm_checks(a, w, y, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, "gemm_mfma")
     if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
@@ -316,7 +319,33 @@ def gemm_mfma(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_scal
         _ptr(a, "a"), a.stride(0), _ptr(w, "w"), rows_w * K, _ptr(y, "y"), dtype_code(y.dtype), y.stride(0),
         M, N, K, _ptr(offsets, "offsets", torch.int32, True), n_groups, _ptr(a_rows, "a_rows", torch.int32, True),
         _ptr(a_scale, "a_scale", torch.float32, True), _ptr(y_rows, "y_rows", torch.int32, True), int(glu),
-        _stream()), "gemm_mfma")
+        int(shape), _stream()), "gemm_mfma")
+
+
+def operand_order(w: torch.Tensor) -> torch.Tensor:
+    """A copy of the matrices ``w[..., N, K]`` (N % 16 == 0, K % 64 == 0) in MFMA operand order:
+    tiles of 16 rows x 32 k, tile (i, j) at ((i * K/32) + j) * 512 elements, inside it
+    W[16i + r][32j + 8q + e] at (q*16 + r) * 8 + e.  Shape and dtype stay as they are."""
+    *lead, N, K = w.shape
+    if N % 16 or K % 64:
+        raise KernelError(f"operand order needs rows a multiple of 16 and columns of 64, got {N} x {K}")
+    n = len(lead)
+    t = w.reshape(*lead, N // 16, 16, K // 32, 4, 8).permute(*range(n), n, n + 2, n + 3, n + 1, n + 4)
+    return t.contiguous().view(*lead, N, K)
+
+
+def gemm_tiled(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None, glu=False,
+               shape=0):
+    """Tiled bf16 MFMA product for many rows over weights in operand order (``operand_order``;
+    see gemm_tiled.hip); arguments as gemm_generic."""
+    rows_w = _gemm_checks(a, w, y, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, "gemm_tiled")
+    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise KernelError(f"gemm_tiled: bfloat16 operands only, got {a.dtype} and {w.dtype}")
+    _check(lib().spite_gemm_tiled(
+        _ptr(a, "a"), a.stride(0), _ptr(w, "w"), rows_w * K, _ptr(y, "y"), dtype_code(y.dtype), y.stride(0),
+        M, N, K, _ptr(offsets, "offsets", torch.int32, True), n_groups, _ptr(a_rows, "a_rows", torch.int32, True),
+        _ptr(a_scale, "a_scale", torch.float32, True), _ptr(y_rows, "y_rows", torch.int32, True), int(glu),
+        int(shape), _stream()), "gemm_tiled")
 
 
 def attn_prefill(q, k_pages, v_pages, out, positions, cu_seqlens, counts, block_table,

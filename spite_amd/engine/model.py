@@ -9,7 +9,7 @@ import torch
 from ..csrc import hipops
 from ..parts import base as P
 from ..parts.base import ParamSpec, PartSpec, CacheNeed
-from ..parts.linear import linear
+from ..parts.linear import linear, Weight
 from .context import Env, Workspace, StepContext, LayerCache
 
 
@@ -58,12 +58,12 @@ class Model:
         if "embed" in tensors:
             self.embed = tensors["embed"].contiguous()
         if "head" in tensors:
-            self.head = tensors["head"].contiguous()
+            self.head = Weight(tensors["head"])
 
     def finish_loading(self):
         if self.embed is None:
             raise RuntimeError("model has no embedding table")
-        if self.spec.head_name is None:
+        if self.spec.head_name is None:       # tied: the table stays row-major, the embedding reads its rows
             self.head = self.embed
 
     def cache_needs(self) -> List[Optional[CacheNeed]]:

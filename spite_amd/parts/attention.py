@@ -15,7 +15,7 @@ import math
 import torch
 
 from .base import Mixer, ParamSpec, CacheNeed, KVNeed, register, build as build_part
-from .linear import linear
+from .linear import linear, Weight
 from ..csrc import hipops
 
 
@@ -53,8 +53,8 @@ class Attention(Mixer):
         # (crates/spite-models/src/llama/llama4.rs:130-139)
         dts = {t[k].dtype for k in ("q_proj", "k_proj", "v_proj")}
         dt = torch.float32 if len(dts) > 1 else dts.pop()
-        self.wqkv = torch.cat([t["q_proj"].to(dt), t["k_proj"].to(dt), t["v_proj"].to(dt)], dim=0).contiguous()
-        self.wo = t["o_proj"].contiguous()
+        self.wqkv = Weight(torch.cat([t["q_proj"].to(dt), t["k_proj"].to(dt), t["v_proj"].to(dt)], dim=0))
+        self.wo = Weight(t["o_proj"])
         self.position.load({k[len("position."):]: v for k, v in t.items() if k.startswith("position.")})
 
     def cache_need(self):

@@ -14,7 +14,7 @@ from __future__ import annotations
 import torch
 
 from .base import FeedForward, ParamSpec, register
-from .linear import linear
+from .linear import linear, Weight
 from ..csrc import hipops
 
 
@@ -32,8 +32,10 @@ class DenseGLU(FeedForward):
 
     def load(self, t):
         dt = t["gate_proj"].dtype if t["gate_proj"].dtype == t["up_proj"].dtype else torch.float32
-        self.w_gate_up = torch.cat([t["gate_proj"].to(dt), t["up_proj"].to(dt)], dim=0).contiguous()
-        self.w_down = t["down_proj"].contiguous()
+        # gate rows then up rows: the up row of a gate row lies F rows further on; in operand order
+        # that needs whole bands, F a multiple of 16
+        self.w_gate_up = Weight(torch.cat([t["gate_proj"].to(dt), t["up_proj"].to(dt)], dim=0), self.F % 16 == 0)
+        self.w_down = Weight(t["down_proj"])
 
     def forward(self, x, x32, ctx):
         T = x.shape[0]
@@ -74,12 +76,12 @@ class MoeTop1Sigmoid(FeedForward):
         sgu = torch.cat([t["shared.gate_proj"], t["shared.up_proj"]], dim=0)
         sdn = t["shared.down_proj"]
         if self.fused_shared and sgu.dtype == gu.dtype and sdn.dtype == dn.dtype:
-            self.w_gate_up = torch.cat([gu, sgu[None]], dim=0).contiguous()
-            self.w_down = torch.cat([dn, sdn[None]], dim=0).contiguous()
+            self.w_gate_up = Weight(torch.cat([gu, sgu[None]], dim=0), self.F % 16 == 0)
+            self.w_down = Weight(torch.cat([dn, sdn[None]], dim=0))
         else:
             self.fused_shared = False
-            self.w_gate_up, self.w_down = gu.contiguous(), dn.contiguous()
-            self.ws_gate_up, self.ws_down = sgu.contiguous(), sdn.contiguous()
+            self.w_gate_up, self.w_down = Weight(gu, self.F % 16 == 0), Weight(dn)
+            self.ws_gate_up, self.ws_down = Weight(sgu, self.Fs % 16 == 0), Weight(sdn)
 
     def forward(self, x, x32, ctx):
         T, E, F, d = x.shape[0], self.E, self.F, self.d

@@ -20,12 +20,31 @@ def _widen(x):
 SKINNY_MAX_ROWS = 64
 
 
+class Weight:
+    """A weight as the product kernels want it.  bfloat16 matrices whose rows are a multiple of
+    16 and whose columns a multiple of 64 are kept in MFMA operand order (``hipops.operand_order``:
+    a wave's operand load is then one run of whole cache lines, which the prefill products are
+    bound by); everything else stays row-major.  ``shape`` is the logical ``[..., out, in]``."""
+
+    __slots__ = ("data", "tiled", "shape", "dtype")
+
+    def __init__(self, w: torch.Tensor, allow_tiled: bool = True):
+        w = w.contiguous()
+        self.shape, self.dtype = tuple(w.shape), w.dtype
+        self.tiled = bool(allow_tiled and w.dtype == torch.bfloat16 and w.dim() >= 2 and w.is_cuda
+                          and w.shape[-2] % 16 == 0 and w.shape[-1] % 64 == 0)
+        self.data = hipops.operand_order(w) if self.tiled else w
+
+
 def linear(x, w, y, *, glu=False, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None, rows=None,
            max_rows=None):
     """y[r] = W . x[r] for ``rows`` rows (default: all of x; for a row list: its length).
 
     With ``glu`` the weight holds gate rows then up rows and y = silu(gate) * up.
     ``max_rows``: the most rows that one group can bring (default: ``rows``)."""
+    tiled = False
+    if isinstance(w, Weight):
+        w, tiled = w.data, w.tiled
     K = x.shape[-1]
     N = y.shape[-1]
     M = rows if rows is not None else x.shape[0]
@@ -33,11 +52,16 @@ def linear(x, w, y, *, glu=False, offsets=None, n_groups=1, a_rows=None, a_scale
     if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and K % 8 == 0 and x.stride(0) % 8 == 0:
         if most <= SKINNY_MAX_ROWS:      # few rows: the time is the weights' stream
             hipops.gemm_skinny(x, w, y, M, N, K, offsets=offsets, n_groups=n_groups, a_rows=a_rows,
-                               a_scale=a_scale, y_rows=y_rows, glu=glu, max_rows=most)
+                               a_scale=a_scale, y_rows=y_rows, glu=glu, max_rows=most, tiled=tiled)
+        elif tiled:
+            hipops.gemm_tiled(x, w, y, M, N, K, offsets=offsets, n_groups=n_groups, a_rows=a_rows, a_scale=a_scale,
+                              y_rows=y_rows, glu=glu)
         else:
             hipops.gemm_mfma(x, w, y, M, N, K, offsets=offsets, n_groups=n_groups, a_rows=a_rows, a_scale=a_scale,
                              y_rows=y_rows, glu=glu)
         return
+    if tiled:
+        raise hipops.KernelError("linear: a weight in operand order met an input that the MFMA products do not take")
     if w.dtype == torch.float32 and x.dtype != torch.float32:
         x32 = _widen(x)
         if y.dtype == torch.float32:

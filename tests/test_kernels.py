@@ -180,6 +180,40 @@ def test_gemm_mfma(M, N, K, out_dtype, glu, grouped):
     run_gemm(ops().gemm_mfma, torch.bfloat16, out_dtype, M, N, K, glu, grouped)
 
 
+# weights in MFMA operand order: rows a multiple of 16, columns of 64
+TILED_SHAPES = [(1, 48, 64), (7, 112, 320), (16, 144, 1088), (64, 80, 512), (33, 528, 192)]
+
+
+@pytest.mark.parametrize("M,N,K", TILED_SHAPES)
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("glu,grouped", [(False, False), (True, False), (False, True), (True, True)])
+@pytest.mark.parametrize("variant", [2, 3, 4, 6, 7])
+def test_gemm_skinny_over_operand_order(M, N, K, out_dtype, glu, grouped, variant):
+    def fn(a, w, y, *args, **kw):
+        ops().gemm_skinny(a, ops().operand_order(w), y, *args, tiled=True, **kw)
+    run_gemm(fn, torch.bfloat16, out_dtype, M, N, K, glu, grouped, variant=variant)
+
+
+@pytest.mark.parametrize("M,N,K", TILED_SHAPES + [(200, 304, 256), (130, 160, 1024), (257, 528, 192), (520, 1040, 128),
+                                                  (300, 64, 448)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("glu,grouped", [(False, False), (True, False), (False, True), (True, True)])
+@pytest.mark.parametrize("shape", [1, 2])
+def test_gemm_tiled(M, N, K, out_dtype, glu, grouped, shape):
+    def fn(a, w, y, *args, **kw):
+        ops().gemm_tiled(a, ops().operand_order(w), y, *args, **kw)
+    run_gemm(fn, torch.bfloat16, out_dtype, M, N, K, glu, grouped, shape=shape)
+
+
+def test_gemm_tiled_refuses_what_it_cannot_do():
+    from spite_amd.csrc.hipops import KernelError
+    a, w, y = rnd(4, 96, dtype=torch.bfloat16), rnd(32, 96, dtype=torch.bfloat16), rnd(4, 32)
+    with pytest.raises(KernelError, match="operand order"):
+        ops().gemm_tiled(a, w, y, 4, 32, 96)
+    with pytest.raises(KernelError, match="operand order"):
+        ops().gemm_skinny(a[:, :72].contiguous(), w[:24, :72].contiguous(), y[:, :24].contiguous(), 4, 24, 72, tiled=True)
+
+
 def test_gemm_skinny_refuses_what_it_cannot_do():
     from spite_amd.csrc.hipops import KernelError
     a, w, y = rnd(2, 12, dtype=torch.bfloat16), rnd(8, 12, dtype=torch.bfloat16), rnd(2, 8)

@@ -81,17 +81,34 @@ def test_loading_binds_every_tensor(tmp_path):
     m = cpu_model(TINY_A)
     load_weights(m, d, torch.float32)
     w = load_file(os.path.join(d, "model.safetensors"))
-    assert torch.equal(m.embed, w["model.embed_tokens.weight"]) and torch.equal(m.head, w["lm_head.weight"])
+    assert torch.equal(m.embed, w["model.embed_tokens.weight"]) and torch.equal(m.head.data, w["lm_head.weight"])
     att = m.blocks[2].mixer
-    assert torch.equal(att.wqkv[:64], w["model.layers.2.self_attn.q_proj.weight"])
-    assert torch.equal(att.wqkv[64:96], w["model.layers.2.self_attn.k_proj.weight"])
+    assert not att.wqkv.tiled                     # operand order is for bfloat16 matrices on the GPU
+    assert torch.equal(att.wqkv.data[:64], w["model.layers.2.self_attn.q_proj.weight"])
+    assert torch.equal(att.wqkv.data[64:96], w["model.layers.2.self_attn.k_proj.weight"])
     ffn = m.blocks[2].ffn
     gu = w["model.layers.2.feed_forward.experts.gate_up_proj"]              # [E, d, 2F]
     assert ffn.w_gate_up.shape == (5, 256, 64)                               # experts + shared, rows gate then up
-    assert torch.equal(ffn.w_gate_up[1, :128], gu[1, :, :128].T) and torch.equal(ffn.w_gate_up[1, 128:], gu[1, :, 128:].T)
-    assert torch.equal(ffn.w_gate_up[4, :128], w["model.layers.2.feed_forward.shared_expert.gate_proj.weight"])
-    assert torch.equal(ffn.w_down[3], w["model.layers.2.feed_forward.experts.down_proj"][3].T)
-    assert torch.equal(ffn.w_down[4], w["model.layers.2.feed_forward.shared_expert.down_proj.weight"])
+    wgu, wdn = ffn.w_gate_up.data, ffn.w_down.data
+    assert torch.equal(wgu[1, :128], gu[1, :, :128].T) and torch.equal(wgu[1, 128:], gu[1, :, 128:].T)
+    assert torch.equal(wgu[4, :128], w["model.layers.2.feed_forward.shared_expert.gate_proj.weight"])
+    assert torch.equal(wdn[3], w["model.layers.2.feed_forward.experts.down_proj"][3].T)
+    assert torch.equal(wdn[4], w["model.layers.2.feed_forward.shared_expert.down_proj.weight"])
+
+
+def test_operand_order_puts_each_lanes_eight_elements_where_the_kernels_read_them():
+    from spite_amd.csrc.hipops import operand_order, KernelError
+    N, K = 48, 128
+    w = torch.arange(2 * N * K, dtype=torch.float32).view(2, N, K)
+    t = operand_order(w).reshape(2, -1)
+    for g, n, k in [(0, 0, 0), (0, 17, 33), (1, 47, 127), (1, 16, 64), (0, 31, 95)]:
+        i, r, j, q, e = n // 16, n % 16, k // 32, (k % 32) // 8, k % 8
+        at = ((i * (K // 32)) + j) * 512 + (q * 16 + r) * 8 + e
+        assert t[g, at] == w[g, n, k]
+    with pytest.raises(KernelError):
+        operand_order(torch.zeros(24, 64))
+    with pytest.raises(KernelError):
+        operand_order(torch.zeros(32, 96))
 
 
 def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
