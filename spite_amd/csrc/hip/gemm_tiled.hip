@@ -129,19 +129,19 @@ void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restri
     // Step u covers 64 k: two half steps t = 2u, 2u+1.  Half step t multiplies W set t % 3
     // with the X tile in LDS buffer u % 2 while W tile t+2 is asked for into set (t+2) % 3.
     // X tile u+1 is asked for at the start of step u and stored to the other LDS buffer at
-    // its end.  Three steps bring every name back; the loop has one way out (leaving it from
-    // the middle made the compiler spill the accumulators), so its last round may run past
-    // the end: only its loads happen then, of the last tile again.
+    // its end.  Three steps bring every name back.  The loop runs whole rounds of three with
+    // no condition inside; up to two steps follow it.  Loads past the end fetch the last tile
+    // again and are never used.
     bf16x8 w0[4], w1[4], w2[4], xr[XL];
     auto step = [&](bf16x8 (&wa)[4], bf16x8 (&wb)[4], bf16x8 (&wc)[4], int u) {
-        // wa: set of half step 2u, wb: of 2u+1, wc: of 2u+2
+        // wa: set of half step 2u, wb: of 2u+1, wc: of 2u+2; wa is loaded again for 2u+3
         load_x(xr, u + 1);
         load_w(wc, 2 * u + 2);
         __builtin_amdgcn_sched_barrier(0);
-        if (u < nu) mul(wa, u & 1, 0);
+        mul(wa, u & 1, 0);
         load_w(wa, 2 * u + 3);
         __builtin_amdgcn_sched_barrier(0);
-        if (u < nu) mul(wb, u & 1, 1);
+        mul(wb, u & 1, 1);
         store_x(xr, (u + 1) & 1);
         __syncthreads();
     };
@@ -150,10 +150,15 @@ void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restri
     load_w(w1, 1);
     store_x(xr, 0);
     __syncthreads();
-    for (int u = 0; u < nu; u += 3) {
+    int u = 0;
+    for (; u + 3 <= nu; u += 3) {
         step(w0, w1, w2, u);            // half steps 0, 1: use w0, w1; load w2 (t=2), w0 (t=3)
         step(w2, w0, w1, u + 1);        // half steps 2, 3: use w2, w0; load w1 (t=4), w2 (t=5)
         step(w1, w2, w0, u + 2);        // half steps 4, 5: use w1, w2; load w0 (t=6), w1 (t=7)
+    }
+    if (u < nu) {
+        step(w0, w1, w2, u);
+        if (u + 1 < nu) step(w2, w0, w1, u + 1);
     }
 
     // acc[a][b][i] of lane (r, q): column ncol[a] + q*4 + i, slot row0 + wm*128 + b*16 + r
@@ -236,7 +241,7 @@ extern "C" int spite_gemm_tiled(const void* X, int ldx, const void* W, long w_gr
     SP_REQUIRE(!offsets || n_groups > 0, "gemm_tiled: grouped call without groups");
     SP_REQUIRE(shape >= 0 && shape <= 2, "gemm_tiled: tile shape %d", shape);
     if (M == 0) return 0;
-    if (shape == 0) shape = (offsets || M <= 128) ? 1 : 2;
+    if (shape == 0) shape = 1;          // measured the faster one at every shape of Llama 4 Scout
     if (shape == 1)
         return launch_tiled<8, 1>(X, ldx, W, w_group_stride, Y, y_dtype, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, st);
     return launch_tiled<4, 2>(X, ldx, W, w_group_stride, Y, y_dtype, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, st);
