@@ -135,76 +135,86 @@ extern "C" int spite_add_rmsnorm(float* h, const float* d1, const float* d2, con
 // the attention kernels read eight consecutive keys of one value column in one load (the
 // layout of an MFMA operand whose sum runs over keys).
 #define SP_MAX_PAIRS 4   // head sizes up to 512
+// Four waves a workgroup; a wave takes `hpw` heads of one token in turn and computes the
+// token's sines and cosines once for all of them.
 template <typename T>
-__global__ void rope_kvwrite_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
-                                    T* __restrict__ k_pages, T* __restrict__ v_pages,
-                                    const int* __restrict__ positions, const int* __restrict__ slot_map,
-                                    const float* __restrict__ inv_freq, int H, int G, int hd, int ps,
-                                    int use_rope, int adjacent, int use_norm, float norm_eps,
-                                    int use_temp, int floor_scale, float attn_scale) {
+__global__ __launch_bounds__(256)
+void rope_kvwrite_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
+                         T* __restrict__ k_pages, T* __restrict__ v_pages,
+                         const int* __restrict__ positions, const int* __restrict__ slot_map,
+                         const float* __restrict__ inv_freq, int H, int G, int hd, int ps,
+                         int use_rope, int adjacent, int use_norm, float norm_eps,
+                         int use_temp, int floor_scale, float attn_scale, int n_heads, int hpw) {
     const int t = blockIdx.x;
-    const int hh = blockIdx.y;
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int half = hd >> 1;
     const int row_w = (H + 2 * G) * hd;
-    const T* src = qkv + (size_t)t * row_w + (size_t)hh * hd;
     const int pos = positions[t];
-    const bool is_q = hh < H;
-    const bool is_v = hh >= H + G;
+    const int slot = slot_map ? slot_map[t] : -1;
+    float sn[SP_MAX_PAIRS], cs[SP_MAX_PAIRS];
+    if (use_rope) {
+#pragma unroll
+        for (int u = 0; u < SP_MAX_PAIRS; ++u) {
+            const int i = lane + u * 64;
+            if (i < half) sincosf((float)pos * inv_freq[i], &sn[u], &cs[u]);
+        }
+    }
+    float temp = 1.f;
+    if (use_temp) temp = logf((float)((pos + 1) / floor_scale) + 1.0f) * attn_scale + 1.0f;
 
-    T* dst;
-    if (is_q) {
-        dst = q_out + ((size_t)t * H + hh) * hd;
-    } else {
-        const int slot = slot_map[t];
-        if (slot < 0) return;
-        const int g = is_v ? hh - H - G : hh - H;
-        const size_t page = slot / ps, off = slot % ps;
-        if (is_v) {
-            T* col = v_pages + (page * G + g) * hd * ps + off;
-            for (int c = lane; c < hd; c += 64) col[(size_t)c * ps] = src[c];
-            return;
-        }
-        dst = k_pages + ((page * G + g) * ps + off) * hd;
-    }
-    float x0[SP_MAX_PAIRS], x1[SP_MAX_PAIRS];
-    float ss = 0.f;
-#pragma unroll
-    for (int u = 0; u < SP_MAX_PAIRS; ++u) {
-        const int i = lane + u * 64;
-        if (i < half) {
-            const int i0 = adjacent ? 2 * i : i;
-            const int i1 = adjacent ? 2 * i + 1 : i + half;
-            float a = to_f32<T>(src[i0]), b = to_f32<T>(src[i1]);
-            if (use_rope) {
-                const float ang = (float)pos * inv_freq[i];
-                float sn, cs;
-                sincosf(ang, &sn, &cs);
-                const float ra = a * cs - b * sn;
-                const float rb = a * sn + b * cs;
-                a = ra; b = rb;
+    for (int it = 0; it < hpw; ++it) {
+        const int hh = blockIdx.y * 4 * hpw + it * 4 + wave;
+        if (hh >= n_heads) break;
+        const T* src = qkv + (size_t)t * row_w + (size_t)hh * hd;
+        const bool is_q = hh < H;
+        const bool is_v = hh >= H + G;
+        T* dst;
+        if (is_q) {
+            dst = q_out + ((size_t)t * H + hh) * hd;
+        } else {
+            if (slot < 0) continue;
+            const int g = is_v ? hh - H - G : hh - H;
+            const size_t page = slot / ps, off = slot % ps;
+            if (is_v) {
+                T* col = v_pages + (page * G + g) * hd * ps + off;
+                for (int c = lane; c < hd; c += 64) col[(size_t)c * ps] = src[c];
+                continue;
             }
-            x0[u] = a; x1[u] = b;
-            ss += a * a + b * b;
+            dst = k_pages + ((page * G + g) * ps + off) * hd;
         }
-    }
-    float scale = 1.f;
-    if (use_norm) {
-        ss = wave_sum(ss);
-        scale = 1.0f / sqrtf(ss / (float)hd + norm_eps);
-    }
-    if (is_q && use_temp) {
-        const int k = (pos + 1) / floor_scale;
-        scale *= logf((float)k + 1.0f) * attn_scale + 1.0f;
-    }
+        float x0[SP_MAX_PAIRS], x1[SP_MAX_PAIRS];
+        float ss = 0.f;
 #pragma unroll
-    for (int u = 0; u < SP_MAX_PAIRS; ++u) {
-        const int i = lane + u * 64;
-        if (i < half) {
-            const int i0 = adjacent ? 2 * i : i;
-            const int i1 = adjacent ? 2 * i + 1 : i + half;
-            dst[i0] = from_f32<T>(x0[u] * scale);
-            dst[i1] = from_f32<T>(x1[u] * scale);
+        for (int u = 0; u < SP_MAX_PAIRS; ++u) {
+            const int i = lane + u * 64;
+            if (i < half) {
+                const int i0 = adjacent ? 2 * i : i;
+                const int i1 = adjacent ? 2 * i + 1 : i + half;
+                float a = to_f32<T>(src[i0]), b = to_f32<T>(src[i1]);
+                if (use_rope) {
+                    const float ra = a * cs[u] - b * sn[u];
+                    const float rb = a * sn[u] + b * cs[u];
+                    a = ra; b = rb;
+                }
+                x0[u] = a; x1[u] = b;
+                ss += a * a + b * b;
+            }
+        }
+        float scale = 1.f;
+        if (use_norm) {
+            ss = wave_sum(ss);
+            scale = 1.0f / sqrtf(ss / (float)hd + norm_eps);
+        }
+        if (is_q) scale *= temp;
+#pragma unroll
+        for (int u = 0; u < SP_MAX_PAIRS; ++u) {
+            const int i = lane + u * 64;
+            if (i < half) {
+                const int i0 = adjacent ? 2 * i : i;
+                const int i1 = adjacent ? 2 * i + 1 : i + half;
+                dst[i0] = from_f32<T>(x0[u] * scale);
+                dst[i1] = from_f32<T>(x1[u] * scale);
+            }
         }
     }
 }
@@ -220,73 +230,108 @@ extern "C" int spite_rope_kvwrite(const void* qkv, void* q_out, void* k_pages, v
     SP_REQUIRE(!use_temp || floor_scale > 0, "rope_kvwrite: floor_scale %d must be >= 1", floor_scale);
     SP_REQUIRE(!use_rope || inv_freq, "rope_kvwrite: rotation needs a frequency table");
     SP_REQUIRE(H + 2 * G <= 65535, "rope_kvwrite: too many heads");
+    SP_REQUIRE(!write_kv || slot_map, "rope_kvwrite: writing the cache needs the rows' slots");
     if (T == 0) return 0;
-    dim3 grid(T, write_kv ? H + 2 * G : H);
+    const int n_heads = write_kv ? H + 2 * G : H;
+    const int hpw = T >= 256 ? 4 : 1;            // many tokens: fewer, longer workgroups
+    dim3 grid(T, (n_heads + 4 * hpw - 1) / (4 * hpw));
     if (dtype == SP_F32)
-        rope_kvwrite_kernel<float><<<grid, 64, 0, st>>>((const float*)qkv, (float*)q_out, (float*)k_pages,
+        rope_kvwrite_kernel<float><<<grid, 256, 0, st>>>((const float*)qkv, (float*)q_out, (float*)k_pages,
             (float*)v_pages, positions, slot_map, inv_freq, H, G, hd, page_size, use_rope, adjacent, use_norm,
-            norm_eps, use_temp, floor_scale, attn_scale);
+            norm_eps, use_temp, floor_scale, attn_scale, n_heads, hpw);
     else if (dtype == SP_BF16)
-        rope_kvwrite_kernel<bf16><<<grid, 64, 0, st>>>((const bf16*)qkv, (bf16*)q_out, (bf16*)k_pages,
+        rope_kvwrite_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)qkv, (bf16*)q_out, (bf16*)k_pages,
             (bf16*)v_pages, positions, slot_map, inv_freq, H, G, hd, page_size, use_rope, adjacent, use_norm,
-            norm_eps, use_temp, floor_scale, attn_scale);
+            norm_eps, use_temp, floor_scale, attn_scale, n_heads, hpw);
     else return sp_fail("rope_kvwrite: unknown dtype %d", dtype);
     SP_LAUNCH_CHECK("rope_kvwrite");
     return 0;
 }
 
 // ------------------------------------------------------------------ top-1 sigmoid router
-// One workgroup per token: logits = W_r . x in fp32, the largest logit wins and the lowest
-// index wins a tie, weight = 1/(1+exp(-logit)).  The token's row sits in LDS; the waves take
-// the experts in turn, a lane's loads are independent 16-byte reads.  A logit's sum runs in
-// an order that depends on the width alone.
+// logits = W_r . x in fp32, the largest logit wins and the lowest index wins a tie,
+// weight = 1/(1+exp(-logit)).  A workgroup takes TB tokens: their rows sit in LDS, the waves
+// take the experts in turn, and a wave reads an expert's row once for all TB tokens (with one
+// token a workgroup the router's matrix would be fetched from L2 once per token, which is
+// what a long prompt's time went into).  A lane's loads are independent 16-byte reads.  A
+// logit's sum runs in an order that depends on the width alone, the same for every TB.
 #define ROUTER_NT 1024
+template <int TB>
 __global__ __launch_bounds__(ROUTER_NT)
 void router_top1_kernel(const float* __restrict__ x, const float* __restrict__ wr,
                         int* __restrict__ expert, float* __restrict__ weight,
-                        float* __restrict__ logits_out, int d, int E) {
-    extern __shared__ float xs[];            // [d] then [E] logits
-    float* lg = xs + d;
-    const int t = blockIdx.x;
+                        float* __restrict__ logits_out, int T, int d, int E) {
+    extern __shared__ float xs[];            // [TB][d] then [TB][E] logits
+    float* lg = xs + (size_t)TB * d;
+    const int t0 = blockIdx.x * TB;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const float* xr = x + (size_t)t * d;
-    for (int c = threadIdx.x; c < d; c += ROUTER_NT) xs[c] = xr[c];
+    for (int u = 0; u < TB; ++u) {
+        const int t = t0 + u < T ? t0 + u : T - 1;          // rows past the end repeat the last one
+        const float* xr = x + (size_t)t * d;
+        for (int c = threadIdx.x; c < d; c += ROUTER_NT) xs[(size_t)u * d + c] = xr[c];
+    }
     __syncthreads();
     const bool vec = (d & 3) == 0 && (((uintptr_t)wr) & 15) == 0;
     for (int e = wave; e < E; e += ROUTER_NT / 64) {
         const float* w = wr + (size_t)e * d;
-        float acc = 0.f;
+        float acc[TB];
+#pragma unroll
+        for (int u = 0; u < TB; ++u) acc[u] = 0.f;
         if (vec) {
             const int nv = d >> 2;
-#pragma unroll 8
+#pragma unroll 4
             for (int c = lane; c < nv; c += 64) {          // independent 16-byte loads, several in flight
                 const f32x4 ww = ((const f32x4*)w)[c];
-                const f32x4 xx = ((const f32x4*)xs)[c];
-                acc += ww[0] * xx[0] + ww[1] * xx[1] + ww[2] * xx[2] + ww[3] * xx[3];
+#pragma unroll
+                for (int u = 0; u < TB; ++u) {
+                    const f32x4 xx = ((const f32x4*)(xs + (size_t)u * d))[c];
+                    acc[u] += ww[0] * xx[0] + ww[1] * xx[1] + ww[2] * xx[2] + ww[3] * xx[3];
+                }
             }
         } else {
-            for (int c = lane; c < d; c += 64) acc += w[c] * xs[c];
+            for (int c = lane; c < d; c += 64) {
+                const float ww = w[c];
+#pragma unroll
+                for (int u = 0; u < TB; ++u) acc[u] += ww * xs[(size_t)u * d + c];
+            }
         }
-        acc = wave_sum(acc);
-        if (lane == 0) lg[e] = acc;
+#pragma unroll
+        for (int u = 0; u < TB; ++u) {
+            const float v = wave_sum(acc[u]);
+            if (lane == 0) lg[u * E + e] = v;
+        }
     }
     __syncthreads();
-    if (logits_out) for (int e = threadIdx.x; e < E; e += ROUTER_NT) logits_out[(size_t)t * E + e] = lg[e];
-    if (threadIdx.x == 0) {
-        float best = lg[0]; int best_e = 0;
-        for (int e = 1; e < E; ++e) if (lg[e] > best) { best = lg[e]; best_e = e; }
-        expert[t] = best_e;
-        weight[t] = 1.0f / (1.0f + expf(-best));
+    if (logits_out)
+        for (int i = threadIdx.x; i < TB * E; i += ROUTER_NT)
+            if (t0 + i / E < T) logits_out[(size_t)(t0 + i / E) * E + i % E] = lg[i];
+    if (threadIdx.x < TB && t0 + threadIdx.x < T) {
+        const float* l = lg + threadIdx.x * E;
+        float best = l[0]; int best_e = 0;
+        for (int e = 1; e < E; ++e) if (l[e] > best) { best = l[e]; best_e = e; }
+        expert[t0 + threadIdx.x] = best_e;
+        weight[t0 + threadIdx.x] = 1.0f / (1.0f + expf(-best));
     }
 }
 
 extern "C" int spite_router_top1(const float* x, const float* wr, int* expert, float* weight,
                                  float* logits_out, int T, int d, int E, hipStream_t st) {
     SP_REQUIRE(T >= 0 && d > 0 && E > 0, "router: bad sizes T=%d d=%d E=%d", T, d, E);
-    const size_t sh = (size_t)(d + E) * sizeof(float);
-    SP_REQUIRE(sh <= 48 * 1024, "router: width %d with %d experts does not fit the kernel's LDS", d, E);
+    const size_t sh1 = (size_t)(d + E) * sizeof(float);
+    SP_REQUIRE(sh1 <= 48 * 1024, "router: width %d with %d experts does not fit the kernel's LDS", d, E);
     if (T == 0) return 0;
-    router_top1_kernel<<<T, ROUTER_NT, sh, st>>>(x, wr, expert, weight, logits_out, d, E);
+    if (T >= 256 && 4 * sh1 <= 150 * 1024) {           // many tokens: four a workgroup
+        static bool allowed = false;
+        if (!allowed) {
+            hipError_t e = hipFuncSetAttribute((const void*)router_top1_kernel<4>,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+            SP_REQUIRE(e == hipSuccess, "router: LDS refused: %s", hipGetErrorString(e));
+            allowed = true;
+        }
+        router_top1_kernel<4><<<(T + 3) / 4, ROUTER_NT, 4 * sh1, st>>>(x, wr, expert, weight, logits_out, T, d, E);
+    } else {
+        router_top1_kernel<1><<<T, ROUTER_NT, sh1, st>>>(x, wr, expert, weight, logits_out, T, d, E);
+    }
     SP_LAUNCH_CHECK("router_top1");
     return 0;
 }
@@ -327,13 +372,59 @@ __global__ void moe_plan_kernel(const int* __restrict__ expert, const float* __r
     }
 }
 
+// The same plan for up to PLAN_MAX_E experts in time linear in T: a workgroup of 256 tokens
+// counts, in LDS, the tokens of every expert in the whole step and among the tokens before its
+// own; a token's slot is then its expert's first slot + the expert's tokens before the
+// workgroup + those before it inside the workgroup.  Counts are integers, so the atomics
+// leave the same list on every run.
+#define PLAN_MAX_E 2048
+__global__ __launch_bounds__(256)
+void moe_plan_hist_kernel(const int* __restrict__ expert, const float* __restrict__ weight,
+                          int* __restrict__ src, float* __restrict__ scale, int* __restrict__ dst,
+                          int* __restrict__ offsets, int T, int E, int shared) {
+    extern __shared__ int sh[];              // total[E], before[E], first[E+1], mine[256]
+    int* total = sh; int* before = sh + E; int* first = sh + 2 * E; int* mine = sh + 3 * E + 1;
+    const int c0 = blockIdx.x * 256, t = c0 + threadIdx.x;
+    for (int e = threadIdx.x; e < 2 * E; e += 256) sh[e] = 0;
+    __syncthreads();
+    for (int j = threadIdx.x; j < T; j += 256) {
+        const int e = expert[j];
+        if ((unsigned)e >= (unsigned)E) continue;       // not a token of any group
+        atomicAdd(&total[e], 1);
+        if (j < c0) atomicAdd(&before[e], 1);
+    }
+    const int me = t < T ? expert[t] : -1;
+    mine[threadIdx.x] = me;
+    __syncthreads();
+    for (int g = threadIdx.x; g <= E; g += 256) {
+        int c = 0;
+        for (int e = 0; e < g; ++e) c += total[e];
+        first[g] = c;
+    }
+    __syncthreads();
+    if (t < T && (unsigned)me < (unsigned)E) {
+        int rank = first[me] + before[me];
+        for (int j = 0; j < (int)threadIdx.x; ++j) rank += mine[j] == me;
+        src[rank] = t; scale[rank] = weight[t]; dst[rank] = t;
+        if (shared) { src[T + t] = t; scale[T + t] = 1.0f; dst[T + t] = T + t; }
+    }
+    if (blockIdx.x == 0) {
+        for (int g = threadIdx.x; g <= E; g += 256) offsets[g] = first[g];
+        if (shared && threadIdx.x == 0) offsets[E + 1] = 2 * T;
+    }
+}
+
 extern "C" int spite_moe_plan(const int* expert, const float* weight, int* src, float* scale, int* dst,
                               int* offsets, int T, int E, int shared, hipStream_t st) {
     SP_REQUIRE(T >= 0 && E > 0 && E < 65535, "moe_plan: bad sizes T=%d E=%d", T, E);
     SP_REQUIRE(T <= 32768, "moe_plan: %d tokens in one step, at most 32768", T);
     const int grid = T > 0 ? (T + 255) / 256 : 1;
-    moe_plan_kernel<<<grid, 256, (size_t)(T > 0 ? T : 1) * sizeof(unsigned short), st>>>(
-        expert, weight, src, scale, dst, offsets, T, E, shared);
+    if (T > 256 && E <= PLAN_MAX_E)
+        moe_plan_hist_kernel<<<grid, 256, (size_t)(3 * E + 1 + 256) * sizeof(int), st>>>(
+            expert, weight, src, scale, dst, offsets, T, E, shared);
+    else
+        moe_plan_kernel<<<grid, 256, (size_t)(T > 0 ? T : 1) * sizeof(unsigned short), st>>>(
+            expert, weight, src, scale, dst, offsets, T, E, shared);
     SP_LAUNCH_CHECK("moe_plan");
     return 0;
 }

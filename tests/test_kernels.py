@@ -67,11 +67,17 @@ def test_add_rmsnorm(d, out_dtype):
 @pytest.mark.parametrize("H,G,hd,adjacent,norm,temp", [(4, 2, 16, False, True, False), (6, 3, 24, False, False, True),
                                                        (5, 1, 64, True, True, True), (8, 8, 128, False, True, False),
                                                        (2, 1, 256, False, True, False)])
-def test_rope_kvwrite(dtype, H, G, hd, adjacent, norm, temp):
-    T, ps, n_pages = 11, 4, 9
+@pytest.mark.parametrize("T", [11, 300])
+def test_rope_kvwrite(dtype, H, G, hd, adjacent, norm, temp, T):
+    ps, n_pages = 4, 9 if T == 11 else 80
     qkv = rnd(T, (H + 2 * G) * hd, dtype=dtype)
-    pos = torch.tensor([3, 4, 5, 0, 1, 2, 3, 40, 41, 42, 7], dtype=torch.int32, device=DEV)
-    slots = torch.tensor([5, 6, 7, 12, 13, 14, 15, 0, 1, 2, 35], dtype=torch.int32, device=DEV)
+    if T == 11:
+        pos = torch.tensor([3, 4, 5, 0, 1, 2, 3, 40, 41, 42, 7], dtype=torch.int32, device=DEV)
+        slots = torch.tensor([5, 6, 7, 12, 13, 14, 15, 0, 1, 2, 35], dtype=torch.int32, device=DEV)
+    else:                                          # many tokens: the kernel's long workgroups
+        g = torch.Generator().manual_seed(T)
+        pos = (torch.arange(T) % 57).to(torch.int32).to(DEV)
+        slots = torch.randperm(n_pages * ps, generator=g)[:T].to(torch.int32).to(DEV)
     inv = plain.rope_inv_freq(hd, 10000.0, None).to(torch.float32).to(DEV)
     q = torch.empty(T, H * hd, dtype=dtype, device=DEV)
     kp = torch.zeros(n_pages, G, ps, hd, dtype=dtype, device=DEV)
@@ -93,7 +99,7 @@ def test_rope_kvwrite(dtype, H, G, hd, adjacent, norm, temp):
         page, off = int(slots[t]) // ps, int(slots[t]) % ps
         assert (kp[page, :, off].double().cpu() - rk[t]).abs().max() < tol
         assert torch.equal(vp[page, :, :, off].cpu().double(), vv[t])
-    written = {(int(s) // ps, int(s) % ps) for s in slots}
+    written = {(int(s) // ps, int(s) % ps) for s in slots.cpu()}
     for p in range(n_pages):
         for o in range(ps):
             if (p, o) not in written:
@@ -430,7 +436,23 @@ def test_attention_refuses_what_it_cannot_do(kind):
 
 
 # ------------------------------------------------------------------ router, expert plan, sampling
-@pytest.mark.parametrize("T,d,E", [(1, 64, 4), (9, 96, 8), (70, 5120, 16), (33, 1000, 128)])
+def test_router_bits_do_not_depend_on_how_many_tokens_a_step_brings():
+    T, d, E = 1029, 520, 16                                 # many tokens share a workgroup; fewer than 256 do not
+    x, wr = rnd(T, d), rnd(E, d, seed=2)
+    out = {}
+    for name, rows in (("all", [(0, T)]), ("pieces", [(0, 200), (200, 455), (455, 456), (456, T)])):
+        expert = torch.empty(T, dtype=torch.int32, device=DEV)
+        weight = torch.empty(T, dtype=torch.float32, device=DEV)
+        logits = torch.empty(T, E, dtype=torch.float32, device=DEV)
+        for b, e in rows:
+            ops().router_top1(x[b:e], wr, expert[b:e], weight[b:e], logits[b:e])
+        out[name] = (expert.cpu(), weight.cpu(), logits.cpu())
+    for a, b in zip(out["all"], out["pieces"]):
+        assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("T,d,E", [(1, 64, 4), (9, 96, 8), (70, 5120, 16), (33, 1000, 128), (300, 512, 16), (1029, 96, 8),
+                                   (2050, 64, 300)])
 def test_router_and_plan(T, d, E):
     x = rnd(T, d)
     wr = rnd(E, d, seed=2)
