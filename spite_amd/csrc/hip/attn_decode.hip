@@ -8,8 +8,12 @@
 //   S^T[keys x heads] = K[keys x hd] . Q^T            (A = K rows as they lie in the page)
 //   O^T[hd x heads]  += V^T[hd x keys] . P^T          (A = value page, stored transposed)
 // The softmax runs down the columns: a lane holds eight keys of one head, the other keys of
-// that head sit in the lanes 16, 32 and 48 further on.  P^T is fed to the second product in
-// the order in which the first one left it; V^T is read in the same order of keys.
+// that head sit in the lanes 16, 32 and 48 further on.  The first product leaves lane (n, qd)
+// with rows qd*4 .. qd*4+3 of each of its two 16-row tiles, the second wants eight consecutive
+// k indices per lane: the rows of the two tiles are therefore the keys qd*8 + i and
+// qd*8 + 4 + i of the block (row r of tile tt is key (r/4)*8 + tt*4 + r%4), so that a lane's
+// eight probabilities belong to eight consecutive keys and its V^T operand is one 16-byte
+// read.
 // Scores, running maximum and sum, and the output are fp32; P is rounded to bf16 only as an
 // MFMA operand.
 #include "common.h"
@@ -62,13 +66,10 @@ void attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_p
         for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
             for (int c = 0; c < NC; ++c)
-                kf[tt][c] = *(const bf16x8*)(kbase + (size_t)(tt * 16 + n) * HD + c * 32 + qd * 8);
-        bf16x4 vf[ND][2];
+                kf[tt][c] = *(const bf16x8*)(kbase + (size_t)((n >> 2) * 8 + tt * 4 + (n & 3)) * HD + c * 32 + qd * 8);
+        bf16x8 vf[ND];
 #pragma unroll
-        for (int d = 0; d < ND; ++d)
-#pragma unroll
-            for (int tt = 0; tt < 2; ++tt)
-                vf[d][tt] = *(const bf16x4*)(vbase + (size_t)(d * 16 + n) * ps + tt * 16 + qd * 4);
+        for (int d = 0; d < ND; ++d) vf[d] = *(const bf16x8*)(vbase + (size_t)(d * 16 + n) * ps + qd * 8);
 
         f32x4 s[2];
 #pragma unroll
@@ -84,7 +85,7 @@ void attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_p
         for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int j = key0 + tt * 16 + qd * 4 + i;
+                const int j = key0 + qd * 8 + tt * 4 + i;
                 ok[tt][i] = j >= lo && j <= p;
                 const float v = ok[tt][i] ? (page < 0 ? NAN : s[tt][i] * scale_log2e) : -INFINITY;
                 s[tt][i] = v;
@@ -110,11 +111,8 @@ void attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_p
         m_run = m_new;
 #pragma unroll
         for (int d = 0; d < ND; ++d) {
-            bf16x8 va;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) { va[e] = vf[d][0][e]; va[4 + e] = vf[d][1][e]; }
             o[d] = o[d] * alpha;
-            o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pf, o[d], 0, 0, 0);
+            o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[d], pf, o[d], 0, 0, 0);
         }
     }
 

@@ -279,8 +279,8 @@ void router_top1_kernel(const float* __restrict__ x, const float* __restrict__ w
         for (int u = 0; u < TB; ++u) acc[u] = 0.f;
         if (vec) {
             const int nv = d >> 2;
-#pragma unroll 4
-            for (int c = lane; c < nv; c += 64) {          // independent 16-byte loads, several in flight
+#pragma unroll 10
+            for (int c = lane; c < nv; c += 64) {          // independent 16-byte loads, ten in flight
                 const f32x4 ww = ((const f32x4*)w)[c];
 #pragma unroll
                 for (int u = 0; u < TB; ++u) {

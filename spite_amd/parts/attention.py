@@ -80,13 +80,15 @@ class Attention(Mixer):
         o = ws.take((T, H * hd), x.dtype)
         if (ctx.decode_only and x.dtype == torch.bfloat16 and hd in (64, 128) and cache.page_size % 32 == 0
                 and H // G <= 16):
-            # split the keys so that about a thousand workgroups run; the bound on the keys is
-            # the block table's width, so the launch is the same for every step of that shape
+            # split the keys so that about five hundred workgroups run (measured: more splits only
+            # add partial results to combine), each wave with at least one block of keys; the
+            # bound on the keys is the block table's width, so the launch is the same for every
+            # step of that shape
             longest = cache.block_table.shape[1] * cache.page_size
             if self.visibility != "full":
                 longest = min(longest, self.span + 32)
             blocks = -(-longest // 32)
-            n_splits = max(1, min(-(-1024 // (T * G)), -(-blocks // 4), 256))
+            n_splits = max(1, min(-(-512 // (T * G)), -(-blocks // 4), 256))
             scratch = ws.take((hipops.attn_decode_workspace(T, H, hd, n_splits) // 4,), torch.float32)
             hipops.attn_decode(q, cache.k_pages, cache.v_pages, o, scratch, ctx.positions, ctx.seq_of_token,
                                cache.block_table, T, H, G, hd, cache.page_size, self.visibility, self.span,
