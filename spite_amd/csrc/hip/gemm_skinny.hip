@@ -204,7 +204,12 @@ extern "C" int spite_gemm_skinny(const void* X, int ldx, const void* W, long w_g
     // measured on MI355X (GB/s of W at Llama 4 Scout's shapes): one row tile per workgroup for
     // the experts' grouped stream, two for the dense projections, four for the output matrix
     if (variant == 0) {
-        if (max_rows <= 16) variant = offsets ? 6 : ((size_t)N * K >= ((size_t)1 << 28) ? 7 : 2);
+        // (with one or two tokens only a few groups have rows at all: more rows of W a workgroup)
+        if (max_rows <= 16) {
+            if (offsets) variant = max_rows <= 2 ? (glu ? 8 : 7) : 6;
+            else if ((size_t)N * K >= ((size_t)1 << 28)) variant = max_rows <= 8 ? 4 : 7;
+            else variant = 8;
+        }
         else variant = max_rows <= 32 ? 2 : 3;
     }
     switch (variant) {

@@ -50,7 +50,9 @@ def linear(x, w, y, *, glu=False, offsets=None, n_groups=1, a_rows=None, a_scale
     M = rows if rows is not None else x.shape[0]
     most = max_rows if max_rows is not None else M
     if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and K % 8 == 0 and x.stride(0) % 8 == 0:
-        if most <= SKINNY_MAX_ROWS:      # few rows: the time is the weights' stream
+        # few rows: the time is the weights' stream (a very tall matrix, the output table, is
+        # streamed faster by the tiled kernel from 33 rows on)
+        if most <= SKINNY_MAX_ROWS and not (tiled and most > 32 and offsets is None and N >= 65536):
             hipops.gemm_skinny(x, w, y, M, N, K, offsets=offsets, n_groups=n_groups, a_rows=a_rows,
                                a_scale=a_scale, y_rows=y_rows, glu=glu, max_rows=most, tiled=tiled)
         elif tiled:
