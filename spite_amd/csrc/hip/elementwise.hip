@@ -35,11 +35,35 @@ extern "C" int spite_embed(const int* ids, const void* table, int dtype, float* 
     return 0;
 }
 
+// ------------------------------------------------------------------ a wave's fp32 dot product
+// sum_c w[c] * xs[c] over a row xs in LDS, by one wave: lane l takes the 16-byte groups l, l+64,
+// ... and the lanes' sums meet in a butterfly.  Every kernel that forms router logits calls
+// this, so a logit has the same bits wherever it is computed; its order of summation depends
+// on the width alone.
+__device__ __forceinline__ float wave_dot_row(const float* __restrict__ w, const float* xs, int d, bool vec, int lane) {
+    float acc = 0.f;
+    if (vec) {
+        const int nv = d >> 2;
+#pragma unroll 10
+        for (int c = lane; c < nv; c += 64) {          // independent 16-byte loads, ten in flight
+            const f32x4 ww = ((const f32x4*)w)[c];
+            const f32x4 xx = ((const f32x4*)xs)[c];
+            acc += ww[0] * xx[0] + ww[1] * xx[1] + ww[2] * xx[2] + ww[3] * xx[3];
+        }
+    } else {
+        for (int c = lane; c < d; c += 64) acc += w[c] * xs[c];
+    }
+    return wave_sum(acc);
+}
+
 // ------------------------------------------------------------------ residual add + RMSNorm
 // v = h[r] + d1[r] + d2[r]; (h[r] = v); out[i] = v * 1/sqrt(mean(v^2)+eps) * w, r = rows ? rows[i] : i.
 // One workgroup of NT threads per row; a thread keeps its elements (groups of four, strided
 // by NT) in registers between the sum and the scaling, so the row is read once.  The sum's
 // order depends on the width alone.
+// With `proj` ([P, d] fp32) the normed fp32 row also goes to LDS and the waves form its P
+// products proj . y into proj_out[i][0..P): the router's logits, without the row going to
+// memory in 32-bit and back.
 #define NORM_NT 512
 #define NORM_MAX_V 8     // widths up to 4*NT*MAX_V = 16384 stay in registers
 template <typename TO, bool VEC>
@@ -47,8 +71,10 @@ __global__ __launch_bounds__(NORM_NT)
 void add_rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ d1,
                         const float* __restrict__ d2, const float* __restrict__ w,
                         TO* __restrict__ out, float* __restrict__ out32,
-                        const int* __restrict__ rows, int d, float eps, int write_h) {
+                        const int* __restrict__ rows, int d, float eps, int write_h,
+                        const float* __restrict__ proj, float* __restrict__ proj_out, int P) {
     __shared__ float red[NORM_NT / 64];
+    extern __shared__ __attribute__((aligned(16))) float ys[];            // [d] if proj
     const int i = blockIdx.x;
     const size_t r = rows ? (size_t)rows[i] : (size_t)i;
     float* hr = h + r * d;
@@ -82,41 +108,56 @@ void add_rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ d1,
 #pragma unroll
                 for (int e = 0; e < 4; ++e) y[e] = v[u][e] * scale * ww[e];
                 if (out32) ((f32x4*)(out32 + (size_t)i * d))[c] = y;
+                if (proj) ((f32x4*)ys)[c] = y;
                 if (out) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) out[(size_t)i * d + 4 * c + e] = from_f32<TO>(y[e]);
                 }
             }
         }
-        return;
+    } else {
+        for (int c = threadIdx.x; c < d; c += NORM_NT) {
+            float x = hr[c];
+            if (a) x += a[c];
+            if (b) x += b[c];
+            if (write_h) hr[c] = x;
+            ss += x * x;
+        }
+        const float ms = block_sum<NORM_NT>(ss, red) / (float)d;
+        const float scale = 1.0f / sqrtf(ms + eps);
+        for (int c = threadIdx.x; c < d; c += NORM_NT) {
+            float x = hr[c];
+            if (!write_h) { if (a) x += a[c]; if (b) x += b[c]; }
+            const float y = x * scale * w[c];
+            if (out) out[(size_t)i * d + c] = from_f32<TO>(y);
+            if (out32) out32[(size_t)i * d + c] = y;
+            if (proj) ys[c] = y;
+        }
     }
-    for (int c = threadIdx.x; c < d; c += NORM_NT) {
-        float x = hr[c];
-        if (a) x += a[c];
-        if (b) x += b[c];
-        if (write_h) hr[c] = x;
-        ss += x * x;
-    }
-    const float ms = block_sum<NORM_NT>(ss, red) / (float)d;
-    const float scale = 1.0f / sqrtf(ms + eps);
-    for (int c = threadIdx.x; c < d; c += NORM_NT) {
-        float x = hr[c];
-        if (!write_h) { if (a) x += a[c]; if (b) x += b[c]; }
-        const float y = x * scale * w[c];
-        if (out) out[(size_t)i * d + c] = from_f32<TO>(y);
-        if (out32) out32[(size_t)i * d + c] = y;
+    if (proj) {
+        __syncthreads();
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+        const bool pvec = (d & 3) == 0 && (((uintptr_t)proj) & 15) == 0;
+        for (int p = wave; p < P; p += NORM_NT / 64) {
+            const float v = wave_dot_row(proj + (size_t)p * d, ys, d, pvec, lane);
+            if (lane == 0) proj_out[(size_t)i * P + p] = v;
+        }
     }
 }
 
 extern "C" int spite_add_rmsnorm(float* h, const float* d1, const float* d2, const float* w, void* out,
                                  int out_dtype, float* out32, const int* rows, int n_rows, int d,
-                                 float eps, int write_h, hipStream_t st) {
+                                 float eps, int write_h, const float* proj, float* proj_out, int P,
+                                 hipStream_t st) {
     SP_REQUIRE(n_rows >= 0 && d > 0 && eps > 0.f, "add_rmsnorm: bad sizes rows=%d d=%d eps=%g", n_rows, d, eps);
+    SP_REQUIRE(!proj || (proj_out && P > 0), "add_rmsnorm: a projection needs its output and size");
+    const size_t sh = proj ? (size_t)d * sizeof(float) : 0;
+    SP_REQUIRE(sh <= 48 * 1024, "add_rmsnorm: rows of %d do not fit the projection's LDS", d);
     if (n_rows == 0) return 0;
     auto al = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
     const bool vec = d % 4 == 0 && d <= 4 * NORM_NT * NORM_MAX_V && al(h) && al(d1) && al(d2) && al(w) && al(out32);
-#define SP_NORM(TO) do { if (vec) add_rmsnorm_kernel<TO, true><<<n_rows, NORM_NT, 0, st>>>(h, d1, d2, w, (TO*)out, out32, rows, d, eps, write_h); \
-        else add_rmsnorm_kernel<TO, false><<<n_rows, NORM_NT, 0, st>>>(h, d1, d2, w, (TO*)out, out32, rows, d, eps, write_h); } while (0)
+#define SP_NORM(TO) do { if (vec) add_rmsnorm_kernel<TO, true><<<n_rows, NORM_NT, sh, st>>>(h, d1, d2, w, (TO*)out, out32, rows, d, eps, write_h, proj, proj_out, P); \
+        else add_rmsnorm_kernel<TO, false><<<n_rows, NORM_NT, sh, st>>>(h, d1, d2, w, (TO*)out, out32, rows, d, eps, write_h, proj, proj_out, P); } while (0)
     if (out_dtype == SP_F32) SP_NORM(float);
     else if (out_dtype == SP_BF16) SP_NORM(bf16);
     else return sp_fail("add_rmsnorm: unknown dtype %d", out_dtype);
@@ -274,13 +315,20 @@ void router_top1_kernel(const float* __restrict__ x, const float* __restrict__ w
     const bool vec = (d & 3) == 0 && (((uintptr_t)wr) & 15) == 0;
     for (int e = wave; e < E; e += ROUTER_NT / 64) {
         const float* w = wr + (size_t)e * d;
+        if (TB == 1) {
+            const float v = wave_dot_row(w, xs, d, vec, lane);
+            if (lane == 0) lg[e] = v;
+            continue;
+        }
+        // TB rows against one read of the expert's row: the same terms in the same order as
+        // wave_dot_row, row by row
         float acc[TB];
 #pragma unroll
         for (int u = 0; u < TB; ++u) acc[u] = 0.f;
         if (vec) {
             const int nv = d >> 2;
 #pragma unroll 10
-            for (int c = lane; c < nv; c += 64) {          // independent 16-byte loads, ten in flight
+            for (int c = lane; c < nv; c += 64) {
                 const f32x4 ww = ((const f32x4*)w)[c];
 #pragma unroll
                 for (int u = 0; u < TB; ++u) {
@@ -343,23 +391,44 @@ extern "C" int spite_router_top1(const float* x, const float* wr, int* expert, f
 //   slots [T,2T) (if shared): src = dst-T = token, scale 1, dst[s] = T + token  (the group E
 //                that every token visits);
 //   offsets[g] = first slot of group g, g in [0, E+1] (+1 with the shared group).
+// With `logits` ([T, E] fp32) the kernels make the router's choice themselves and write it to
+// expert[] and weight[]: the largest logit, the lowest index among equals, weight =
+// 1/(1+exp(-logit)).
+__device__ __forceinline__ int top1_of(const float* __restrict__ l, int E, float* best_out) {
+    float best = l[0]; int best_e = 0;
+    for (int e = 1; e < E; ++e) { const float v = l[e]; if (v > best) { best = v; best_e = e; } }
+    if (best_out) *best_out = best;
+    return best_e;
+}
+
 // Each thread ranks one token by counting over all tokens in shared memory: no atomics, the
 // order is the same on every run.
-__global__ void moe_plan_kernel(const int* __restrict__ expert, const float* __restrict__ weight,
+__global__ void moe_plan_kernel(int* __restrict__ expert, float* __restrict__ weight,
+                                const float* __restrict__ logits,
                                 int* __restrict__ src, float* __restrict__ scale, int* __restrict__ dst,
                                 int* __restrict__ offsets, int T, int E, int shared) {
     extern __shared__ unsigned short e_of[];
-    for (int i = threadIdx.x; i < T; i += blockDim.x) e_of[i] = (unsigned short)expert[i];
+    for (int i = threadIdx.x; i < T; i += blockDim.x)
+        e_of[i] = (unsigned short)(logits ? top1_of(logits + (size_t)i * E, E, nullptr) : expert[i]);
     __syncthreads();
     const int t = blockIdx.x * blockDim.x + threadIdx.x;
     if (t < T) {
         const int me = e_of[t];
+        float wt;
+        if (logits) {
+            float best;
+            top1_of(logits + (size_t)t * E, E, &best);
+            wt = 1.0f / (1.0f + expf(-best));
+            expert[t] = me; weight[t] = wt;
+        } else {
+            wt = weight[t];
+        }
         int rank = 0;
         for (int j = 0; j < T; ++j) {
             const int ej = e_of[j];
             rank += (ej < me) || (ej == me && j < t);
         }
-        src[rank] = t; scale[rank] = weight[t]; dst[rank] = t;
+        src[rank] = t; scale[rank] = wt; dst[rank] = t;
         if (shared) { src[T + t] = t; scale[T + t] = 1.0f; dst[T + t] = T + t; }
     }
     if (blockIdx.x == 0) {
@@ -379,7 +448,8 @@ __global__ void moe_plan_kernel(const int* __restrict__ expert, const float* __r
 // leave the same list on every run.
 #define PLAN_MAX_E 2048
 __global__ __launch_bounds__(256)
-void moe_plan_hist_kernel(const int* __restrict__ expert, const float* __restrict__ weight,
+void moe_plan_hist_kernel(int* __restrict__ expert, float* __restrict__ weight,
+                          const float* __restrict__ logits,
                           int* __restrict__ src, float* __restrict__ scale, int* __restrict__ dst,
                           int* __restrict__ offsets, int T, int E, int shared) {
     extern __shared__ int sh[];              // total[E], before[E], first[E+1], mine[256]
@@ -388,12 +458,23 @@ void moe_plan_hist_kernel(const int* __restrict__ expert, const float* __restric
     for (int e = threadIdx.x; e < 2 * E; e += 256) sh[e] = 0;
     __syncthreads();
     for (int j = threadIdx.x; j < T; j += 256) {
-        const int e = expert[j];
+        const int e = logits ? top1_of(logits + (size_t)j * E, E, nullptr) : expert[j];
         if ((unsigned)e >= (unsigned)E) continue;       // not a token of any group
         atomicAdd(&total[e], 1);
         if (j < c0) atomicAdd(&before[e], 1);
     }
-    const int me = t < T ? expert[t] : -1;
+    int me = -1;
+    float wt = 0.f;
+    if (t < T) {
+        if (logits) {
+            float best;
+            me = top1_of(logits + (size_t)t * E, E, &best);
+            wt = 1.0f / (1.0f + expf(-best));
+            expert[t] = me; weight[t] = wt;
+        } else {
+            me = expert[t]; wt = weight[t];
+        }
+    }
     mine[threadIdx.x] = me;
     __syncthreads();
     for (int g = threadIdx.x; g <= E; g += 256) {
@@ -405,7 +486,7 @@ void moe_plan_hist_kernel(const int* __restrict__ expert, const float* __restric
     if (t < T && (unsigned)me < (unsigned)E) {
         int rank = first[me] + before[me];
         for (int j = 0; j < (int)threadIdx.x; ++j) rank += mine[j] == me;
-        src[rank] = t; scale[rank] = weight[t]; dst[rank] = t;
+        src[rank] = t; scale[rank] = wt; dst[rank] = t;
         if (shared) { src[T + t] = t; scale[T + t] = 1.0f; dst[T + t] = T + t; }
     }
     if (blockIdx.x == 0) {
@@ -414,17 +495,18 @@ void moe_plan_hist_kernel(const int* __restrict__ expert, const float* __restric
     }
 }
 
-extern "C" int spite_moe_plan(const int* expert, const float* weight, int* src, float* scale, int* dst,
+// `logits` null: expert[] and weight[] are inputs; else they are outputs.
+extern "C" int spite_moe_plan(int* expert, float* weight, const float* logits, int* src, float* scale, int* dst,
                               int* offsets, int T, int E, int shared, hipStream_t st) {
     SP_REQUIRE(T >= 0 && E > 0 && E < 65535, "moe_plan: bad sizes T=%d E=%d", T, E);
     SP_REQUIRE(T <= 32768, "moe_plan: %d tokens in one step, at most 32768", T);
     const int grid = T > 0 ? (T + 255) / 256 : 1;
     if (T > 256 && E <= PLAN_MAX_E)
         moe_plan_hist_kernel<<<grid, 256, (size_t)(3 * E + 1 + 256) * sizeof(int), st>>>(
-            expert, weight, src, scale, dst, offsets, T, E, shared);
+            expert, weight, logits, src, scale, dst, offsets, T, E, shared);
     else
         moe_plan_kernel<<<grid, 256, (size_t)(T > 0 ? T : 1) * sizeof(unsigned short), st>>>(
-            expert, weight, src, scale, dst, offsets, T, E, shared);
+            expert, weight, logits, src, scale, dst, offsets, T, E, shared);
     SP_LAUNCH_CHECK("moe_plan");
     return 0;
 }

@@ -34,10 +34,10 @@ def lib():
         P, I, L, F = c_void_p, c_int, c_long, c_float
         sigs = {
             "spite_embed": [P, P, I, P, I, I, I, P],
-            "spite_add_rmsnorm": [P, P, P, P, P, I, P, P, I, I, F, I, P],
+            "spite_add_rmsnorm": [P, P, P, P, P, I, P, P, I, I, F, I, P, P, I, P],
             "spite_rope_kvwrite": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, I, I, F, I, P],
             "spite_router_top1": [P, P, P, P, P, I, I, I, P],
-            "spite_moe_plan": [P, P, P, P, P, P, I, I, I, P],
+            "spite_moe_plan": [P, P, P, P, P, P, P, I, I, I, P],
             "spite_convert": [P, I, P, I, c_size_t, P],
             "spite_gemm_generic": [P, I, P, L, I, P, I, I, I, I, I, P, I, P, P, P, I, P],
             "spite_attn_generic": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, P],
@@ -106,9 +106,12 @@ def embed(ids, table, h):
                              _ptr(h, "h", torch.float32), T, d, table.shape[0], _stream()), "embed")
 
 
-def add_rmsnorm(h, w, eps, out=None, out32=None, d1=None, d2=None, rows=None, n_rows=None, write_h=True):
+def add_rmsnorm(h, w, eps, out=None, out32=None, d1=None, d2=None, rows=None, n_rows=None, write_h=True,
+                proj=None, proj_out=None):
     """v = h[r] + d1[r] + d2[r] (stored back if write_h); out[i] = rmsnorm(v) * w with r =
-    rows[i] or i.  h, d1, d2, out32 fp32; w fp32 [d]; out fp32 or bf16."""
+    rows[i] or i.  h, d1, d2, out32 fp32; w fp32 [d]; out fp32 or bf16.  With ``proj`` ([P, d]
+    fp32) also proj_out[i] = proj . (the normed row in fp32), [n, P] fp32: the same bits as
+    ``router_top1`` gives for that row."""
     d = h.shape[-1]
     n = n_rows if n_rows is not None else (rows.numel() if rows is not None else h.shape[0])
     for name, t in (("d1", d1), ("d2", d2)):
@@ -121,11 +124,19 @@ def add_rmsnorm(h, w, eps, out=None, out32=None, d1=None, d2=None, rows=None, n_
             raise KernelError(f"add_rmsnorm: {name} {tuple(t.shape)} is too small for {n} rows of {d}")
     if rows is None and n > h.shape[0]:
         raise KernelError("add_rmsnorm: more rows asked than h holds")
+    P = 0
+    if proj is not None:
+        P = proj.shape[0]
+        if proj.dim() != 2 or proj.shape[1] != d or proj_out is None or proj_out.dim() != 2 \
+                or proj_out.shape[0] < n or proj_out.shape[1] != P:
+            raise KernelError("add_rmsnorm: projection [P, d] with an output [rows, P]")
     _check(lib().spite_add_rmsnorm(
         _ptr(h, "h", torch.float32), _ptr(d1, "d1", torch.float32, True), _ptr(d2, "d2", torch.float32, True),
         _ptr(w, "w", torch.float32), _ptr(out, "out", None, True),
         dtype_code(out.dtype) if out is not None else F32, _ptr(out32, "out32", torch.float32, True),
-        _ptr(rows, "rows", torch.int32, True), n, d, float(eps), int(write_h), _stream()), "add_rmsnorm")
+        _ptr(rows, "rows", torch.int32, True), n, d, float(eps), int(write_h),
+        _ptr(proj, "proj", torch.float32, True), _ptr(proj_out, "proj_out", torch.float32, True), P, _stream()),
+        "add_rmsnorm")
 
 
 def rope_kvwrite(qkv, q_out, k_pages, v_pages, positions, slot_map, inv_freq, H, G, hd, page_size, *,
@@ -167,15 +178,18 @@ def router_top1(x32, w_router, expert, weight, logits_out=None):
            "router_top1")
 
 
-def moe_plan(expert, weight, src, scale, dst, offsets, T, E, shared):
-    """Row list of the grouped products from the router's choice (see the kernel)."""
+def moe_plan(expert, weight, src, scale, dst, offsets, T, E, shared, logits=None):
+    """Row list of the grouped products from the router's choice (see the kernel).  With
+    ``logits`` ([T, E] fp32) the choice is made here and written to ``expert`` and ``weight``."""
     n = 2 * T if shared else T
     if src.numel() < n or scale.numel() < n or dst.numel() < n or offsets.numel() < E + 1 + int(bool(shared)):
         raise KernelError("moe_plan: output arrays too small")
     if expert.numel() < T or weight.numel() < T:
         raise KernelError("moe_plan: inputs too small")
+    if logits is not None and (logits.dim() != 2 or logits.shape[0] < T or logits.shape[1] != E):
+        raise KernelError(f"moe_plan: logits {tuple(logits.shape)} for {T} tokens and {E} experts")
     _check(lib().spite_moe_plan(_ptr(expert, "expert", torch.int32), _ptr(weight, "weight", torch.float32),
-                                _ptr(src, "src", torch.int32), _ptr(scale, "scale", torch.float32),
+                                _ptr(logits, "logits", torch.float32, True), _ptr(src, "src", torch.int32), _ptr(scale, "scale", torch.float32),
                                 _ptr(dst, "dst", torch.int32), _ptr(offsets, "offsets", torch.int32),
                                 T, E, int(bool(shared)), _stream()), "moe_plan")
 

@@ -100,6 +100,10 @@ class Part:
 
 
 class Norm(Part):
+    #: True when forward() takes ``proj`` / ``proj_out``: a small fp32 matrix [P, d] whose
+    #: products with the normed fp32 rows are formed in the same pass (router logits)
+    projects = False
+
     def forward(self, h, out, *, d1=None, d2=None, out32=None, rows=None, write_h=True) -> None:
         """h (fp32 [T,d]) += d1 + d2 (kept if write_h); out[i] (and out32[i]) = norm(h[r]), r =
         rows[i] or i."""
@@ -132,7 +136,13 @@ class FeedForward(Part):
     #: ask the block for the normed input in fp32 as well (routers want it)
     wants_f32_input = False
 
-    def forward(self, x, x32, ctx):
+    def input_projection(self):
+        """An fp32 matrix [P, d] whose products with the fp32 normed input this part wants
+        (router logits), or None.  A block whose norm ``projects`` then calls
+        ``forward(x, None, ctx, projected=logits)`` instead of handing over x32."""
+        return None
+
+    def forward(self, x, x32, ctx, projected=None):
         """x [T,d] (x32: the same in fp32, if asked for) -> a tuple of one or two fp32 [T,d]
         increments of the residual, taken from ``ctx.ws``."""
         raise NotImplementedError

@@ -32,6 +32,12 @@ class PreNormBlock(Block):
         self.norm1.forward(h, n, d1=d1, d2=d2)
         delta = self.mixer.forward(n, ctx, cache)
         n2 = ws.take((T, d), self.env.dtype)
+        proj = self.ffn.input_projection() if self.norm2.projects else None
+        if proj is not None and proj.shape[1] * 4 <= 48 * 1024:
+            # the norm forms the feed-forward's small fp32 products (router logits) itself
+            logits = ws.take((T, proj.shape[0]), torch.float32)
+            self.norm2.forward(h, n2, d1=delta, proj=proj, proj_out=logits)
+            return tuple(self.ffn.forward(n2, None, ctx, projected=logits))
         n2_32 = None
         if self.ffn.wants_f32_input:
             n2_32 = n2 if n2.dtype == torch.float32 else ws.take((T, d), torch.float32)

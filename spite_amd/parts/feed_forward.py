@@ -37,7 +37,7 @@ class DenseGLU(FeedForward):
         self.w_gate_up = Weight(torch.cat([t["gate_proj"].to(dt), t["up_proj"].to(dt)], dim=0), self.F % 16 == 0)
         self.w_down = Weight(t["down_proj"])
 
-    def forward(self, x, x32, ctx):
+    def forward(self, x, x32, ctx, projected=None):
         T = x.shape[0]
         act = ctx.ws.take((T, self.F), x.dtype)
         linear(x, self.w_gate_up, act, glu=True)
@@ -83,20 +83,26 @@ class MoeTop1Sigmoid(FeedForward):
             self.w_gate_up, self.w_down = Weight(gu, self.F % 16 == 0), Weight(dn)
             self.ws_gate_up, self.ws_down = Weight(sgu, self.Fs % 16 == 0), Weight(sdn)
 
-    def forward(self, x, x32, ctx):
+    def input_projection(self):
+        return self.w_router if self.w_router is not None and self.w_router.dtype == torch.float32 else None
+
+    def forward(self, x, x32, ctx, projected=None):
+        """``projected``: the router's logits [T, E] if the block's norm formed them; else they
+        are computed here from x32."""
         T, E, F, d = x.shape[0], self.E, self.F, self.d
         ws = ctx.ws
         expert = ws.take((T,), torch.int32)
         weight = ws.take((T,), torch.float32)
-        hipops.router_top1(x32, self.w_router, expert, weight)
-        if ctx.extras.get("trace") is not None:      # a testing aid: which expert each row took
-            ctx.extras["trace"].setdefault("moe_experts", []).append(expert.clone())
+        if projected is None:
+            hipops.router_top1(x32, self.w_router, expert, weight)
         n = 2 * T if self.fused_shared else T
         src, dst = ws.take((n,), torch.int32), ws.take((n,), torch.int32)
         scale = ws.take((n,), torch.float32)
         groups = E + 1 if self.fused_shared else E
         offsets = ws.take((groups + 1,), torch.int32)
-        hipops.moe_plan(expert, weight, src, scale, dst, offsets, T, E, self.fused_shared)
+        hipops.moe_plan(expert, weight, src, scale, dst, offsets, T, E, self.fused_shared, logits=projected)
+        if ctx.extras.get("trace") is not None:      # a testing aid: which expert each row took
+            ctx.extras["trace"].setdefault("moe_experts", []).append(expert.clone())
         act = ws.take((n, F), x.dtype)
         linear(x, self.w_gate_up, act, glu=True, offsets=offsets, n_groups=groups, a_rows=src, a_scale=scale, rows=n,
                max_rows=T)

@@ -9,6 +9,7 @@ from ..csrc import hipops
 @register("norm", "rms")
 class RMSNorm(Norm):
     graph_safe = True
+    projects = True
 
     def __init__(self, env, width: int, eps: float):
         self.width = int(width)
@@ -21,6 +22,7 @@ class RMSNorm(Norm):
     def load(self, tensors):
         self.weight = tensors["weight"]
 
-    def forward(self, h, out, *, d1=None, d2=None, out32=None, rows=None, write_h=True):
+    def forward(self, h, out, *, d1=None, d2=None, out32=None, rows=None, write_h=True, proj=None, proj_out=None):
         hipops.add_rmsnorm(h, self.weight, self.eps, out=out, out32=out32, d1=d1, d2=d2, rows=rows,
-                           n_rows=(rows.numel() if rows is not None else h.shape[0]), write_h=write_h)
+                           n_rows=(rows.numel() if rows is not None else h.shape[0]), write_h=write_h,
+                           proj=proj, proj_out=proj_out)

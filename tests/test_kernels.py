@@ -436,6 +436,39 @@ def test_attention_refuses_what_it_cannot_do(kind):
 
 
 # ------------------------------------------------------------------ router, expert plan, sampling
+@pytest.mark.parametrize("T,d,E", [(1, 64, 4), (9, 5120, 16), (300, 96, 8), (70, 1002, 128), (1029, 520, 16)])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_norm_with_projection_and_plan_from_logits_match_the_router(T, d, E, out_dtype):
+    # the norm forms the router's logits in its own pass and the plan kernel takes the choice from
+    # them: the same bits as the three kernels in a row give
+    h = rnd(T, d, seed=5)
+    delta = rnd(T, d, seed=6)
+    w, wr = rnd(d, seed=7) + 1.0, rnd(E, d, seed=8)
+    wr[3 % E] = wr[1 % E]
+    out_a, out_b = torch.empty(T, d, dtype=out_dtype, device=DEV), torch.empty(T, d, dtype=out_dtype, device=DEV)
+    x32 = torch.empty(T, d, device=DEV)
+    h_a, h_b = h.clone(), h.clone()
+    ops().add_rmsnorm(h_a, w, 1e-5, out=out_a, out32=x32, d1=delta)
+    expert_a = torch.empty(T, dtype=torch.int32, device=DEV)
+    weight_a = torch.empty(T, device=DEV)
+    logits_a = torch.empty(T, E, device=DEV)
+    ops().router_top1(x32, wr, expert_a, weight_a, logits_a)
+    logits_b = torch.empty(T, E, device=DEV)
+    ops().add_rmsnorm(h_b, w, 1e-5, out=out_b, d1=delta, proj=wr, proj_out=logits_b)
+    assert torch.equal(h_a, h_b) and torch.equal(out_a, out_b) and torch.equal(logits_a, logits_b)
+    n = 2 * T
+    plans = []
+    for logits in (None, logits_b):
+        expert = expert_a.clone() if logits is None else torch.full((T,), -7, dtype=torch.int32, device=DEV)
+        weight = weight_a.clone() if logits is None else torch.zeros(T, device=DEV)
+        src, dst = torch.empty(n, dtype=torch.int32, device=DEV), torch.empty(n, dtype=torch.int32, device=DEV)
+        scale, offsets = torch.empty(n, device=DEV), torch.empty(E + 2, dtype=torch.int32, device=DEV)
+        ops().moe_plan(expert, weight, src, scale, dst, offsets, T, E, True, logits=logits)
+        plans.append((expert, weight, src, dst, scale, offsets))
+    for a, b in zip(*plans):
+        assert torch.equal(a, b)
+
+
 def test_router_bits_do_not_depend_on_how_many_tokens_a_step_brings():
     T, d, E = 1029, 520, 16                                 # many tokens share a workgroup; fewer than 256 do not
     x, wr = rnd(T, d), rnd(E, d, seed=2)
