@@ -210,7 +210,7 @@ extern "C" int spite_gemm_skinny(const void* X, int ldx, const void* W, long w_g
             else if ((size_t)N * K >= ((size_t)1 << 28)) variant = max_rows <= 8 ? 4 : 7;
             else variant = 8;
         }
-        else variant = max_rows <= 32 ? 2 : 3;
+        else variant = max_rows <= 32 ? 2 : (offsets ? 3 : 9);
     }
     switch (variant) {
         case 1: return launch_skinny<1, 1, 4, 8>(SP_ARGS);
@@ -221,6 +221,7 @@ extern "C" int spite_gemm_skinny(const void* X, int ldx, const void* W, long w_g
         case 6: return launch_skinny<1, 1, 2, 8>(SP_ARGS);
         case 7: return launch_skinny<4, 1, 2, 8>(SP_ARGS);
         case 8: return launch_skinny<2, 1, 2, 8>(SP_ARGS);
+        case 9: return launch_skinny<2, 4, 2, 8>(SP_ARGS);
         default: return sp_fail("gemm_skinny: unknown variant %d", variant);
     }
 #undef SP_ARGS

@@ -174,7 +174,7 @@ def test_gemm_generic(M, N, K, dtype, out_dtype, glu, grouped):
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES + [(3, 40, 8), (12, 16, 4104)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("glu,grouped", [(False, False), (True, False), (False, True), (True, True)])
-@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8, 9])
 def test_gemm_skinny(M, N, K, out_dtype, glu, grouped, variant):
     run_gemm(ops().gemm_skinny, torch.bfloat16, out_dtype, M, N, K, glu, grouped, variant=variant)
 
@@ -193,7 +193,7 @@ TILED_SHAPES = [(1, 48, 64), (7, 112, 320), (16, 144, 1088), (64, 80, 512), (33,
 @pytest.mark.parametrize("M,N,K", TILED_SHAPES)
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("glu,grouped", [(False, False), (True, False), (False, True), (True, True)])
-@pytest.mark.parametrize("variant", [2, 3, 4, 6, 7])
+@pytest.mark.parametrize("variant", [2, 3, 4, 6, 7, 8, 9])
 def test_gemm_skinny_over_operand_order(M, N, K, out_dtype, glu, grouped, variant):
     def fn(a, w, y, *args, **kw):
         ops().gemm_skinny(a, ops().operand_order(w), y, *args, tiled=True, **kw)
