@@ -32,7 +32,16 @@ TINY_B = dict(
                       original_max_position_embeddings=64),
     attention_chunk_size=16, use_qk_norm=False, attn_temperature_tuning=False,
     tie_word_embeddings=False, torch_dtype="float32")
-CONFIGS = {"A": TINY_A, "B": TINY_B}
+# sizes that the MFMA kernels take (head size 64, pages of 32 keys, widths in operand order):
+# the replay tests then run the kernels that serving runs, not their generic stand-ins
+TINY_C = dict(
+    architectures=["Llama4ForCausalLM"], num_hidden_layers=4, hidden_size=128, num_attention_heads=6,
+    num_key_value_heads=2, head_dim=64, rms_norm_eps=1e-5, num_local_experts=4, num_experts_per_tok=1,
+    intermediate_size=128, intermediate_size_mlp=192, interleave_moe_layer_step=1, vocab_size=400,
+    rope_theta=50000.0, rope_scaling=None, attention_chunk_size=64, no_rope_layers=[1, 0, 1, 1],
+    use_qk_norm=True, attn_temperature_tuning=True, floor_scale=32, attn_scale=0.2,
+    tie_word_embeddings=False, torch_dtype="float32")
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
 
 
 def planted_tensors(cfg: dict, seed: int, std: float = 0.05, qk_gain: float = 2.0, router_gain: float = 8.0):

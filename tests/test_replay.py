@@ -31,8 +31,9 @@ HINT_REL = TOL_BF16_REL
 REQUESTS = {
     "A": {"a0": 5 + 16, "a1": 23 + 16, "a2": 40 + 16, "a3": 131},
     "B": {"b0": 1 + 16, "b1": 7 + 16, "b2": 16 + 16, "b3": 33 + 16, "b4": 70 + 16},
+    "C": {"c0": 5 + 16, "c1": 70, "c2": 150, "c3": 300},
 }
-PAGE = {"A": 16, "B": 8}
+PAGE = {"A": 16, "B": 8, "C": 32}
 
 
 class Case:
@@ -48,6 +49,8 @@ class Case:
         self.tol = TOL_F32 if dtype == "float32" else TOL_BF16_REL * self.scale
         self.results = {}
         self.Engine = Engine
+        # a pool for one request at a time, whole
+        self.pool = max(256, -(-max(len(t) for t in self.reqs.values()) // PAGE[name]) * PAGE[name])
 
     def engine(self, cache_tokens, page_size=None, max_requests=4):
         return self.Engine(self.dir, dtype=self.dtype, page_size=page_size or PAGE[self.name],
@@ -76,7 +79,7 @@ class Case:
         return ref
 
 
-@pytest.fixture(scope="module", params=[("A", "float32"), ("B", "float32"), ("A", "bfloat16"), ("B", "bfloat16")],
+@pytest.fixture(scope="module", params=[("A", "float32"), ("B", "float32"), ("A", "bfloat16"), ("B", "bfloat16"), ("C", "bfloat16")],
                 ids=lambda p: f"{p[0]}-{p[1]}")
 def case(request, tmp_path_factory):
     return Case(*request.param, tmp_path_factory.mktemp("replay"))
@@ -92,17 +95,17 @@ def check(case, result, label, reqs=None):
 
 
 def test_whole(case):
-    check(case, case.replay(H.schedule_whole(case.reqs), 256), "whole")
+    check(case, case.replay(H.schedule_whole(case.reqs), case.pool), "whole")
 
 
 def test_last_32_one_by_one(case):
-    check(case, case.replay(H.schedule_tail_one_by_one(case.reqs), 256), "tail")
+    check(case, case.replay(H.schedule_tail_one_by_one(case.reqs), case.pool), "tail")
 
 
 def test_portions_of_changing_size(case):
     steps = H.schedule_portions(case.reqs)
     assert min(len(e["tokens"]) for s in steps for e in s["entries"]) <= 2
-    check(case, case.replay(steps, 256), "portions")
+    check(case, case.replay(steps, case.pool), "portions")
 
 
 def test_mixed_with_pages_used_again(case):
@@ -184,7 +187,7 @@ def test_faults_are_visible(case):
     the reference's sliding window in place of chunks, or with one expert swapped, differs
     from the right logits by far more than the tolerance."""
     import plain_llama4 as plain
-    rid = "a3" if case.name == "A" else "b4"
+    rid = {"A": "a3", "B": "b4", "C": "c3"}[case.name]
     toks = case.reqs[rid]
     right = np.stack([case.plain[(rid, i)] for i in range(len(toks))])
     window = plain.forward(case.cfg, case.weights, toks, visibility="window").numpy()
