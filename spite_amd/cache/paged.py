@@ -16,7 +16,7 @@ from typing import Dict, List, Optional, Sequence
 import numpy as np
 import torch
 
-from ..csrc import hostlib
+from ..csrc import hostlib, hipops
 from ..parts.base import CacheNeed
 
 _KINDS = {"full": 0, "chunk": 1, "window": 2}
@@ -181,6 +181,12 @@ class PagedCache:
 
     def table_len(self, slot, g) -> int:
         return int(self._lib.spc_table_len(self._h, slot, g))
+
+    def kv_tiled(self, cache_id: int) -> bool:
+        """Whether this cache's pages are kept in the MFMA attention kernels' operand order
+        (bfloat16, head size and page size multiples of 32) rather than row-major."""
+        g = self.groups[self._group_of[cache_id]]
+        return hipops.kv_tiled_ok(self.dtype, g.key[1], self.page_size)
 
     def layer_pages(self, cache_id: int):
         g = self.groups[self._group_of[cache_id]]

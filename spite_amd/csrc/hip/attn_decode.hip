@@ -13,7 +13,9 @@
 // k indices per lane: the rows of the two tiles are therefore the keys qd*8 + i and
 // qd*8 + 4 + i of the block (row r of tile tt is key (r/4)*8 + tt*4 + r%4), so that a lane's
 // eight probabilities belong to eight consecutive keys and its V^T operand is one 16-byte
-// read.
+// read.  The pages hold keys and values in that operand order (see common.h), tile by tile, so
+// that every load of a wave is one kilobyte in a row; the cache is read once, with
+// non-temporal loads.
 // Scores, running maximum and sum, and the output are fp32; P is rounded to bf16 only as an
 // MFMA operand.
 #include "common.h"
@@ -59,17 +61,18 @@ void attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_p
         const int page = bt[key0 / ps];
         const int off0 = key0 % ps;
         const size_t pg = (size_t)(page < 0 ? 0 : page) * G + g;
-        const bf16* kbase = k_pages + (pg * ps + off0) * HD;
-        const bf16* vbase = v_pages + pg * HD * ps + off0;
+        const int blk = off0 >> 5;                                   // the block of 32 keys inside the page
+        const bf16* kbase = k_pages + pg * ps * HD + (size_t)blk * 2 * NC * 512 + lane * 8;
+        const bf16* vbase = v_pages + pg * HD * ps + (size_t)blk * ND * 512 + lane * 8;
         bf16x8 kf[2][NC];
 #pragma unroll
         for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
             for (int c = 0; c < NC; ++c)
-                kf[tt][c] = *(const bf16x8*)(kbase + (size_t)((n >> 2) * 8 + tt * 4 + (n & 3)) * HD + c * 32 + qd * 8);
+                kf[tt][c] = __builtin_nontemporal_load((const bf16x8*)(kbase + (tt * NC + c) * 512));
         bf16x8 vf[ND];
 #pragma unroll
-        for (int d = 0; d < ND; ++d) vf[d] = *(const bf16x8*)(vbase + (size_t)(d * 16 + n) * ps + qd * 8);
+        for (int d = 0; d < ND; ++d) vf[d] = __builtin_nontemporal_load((const bf16x8*)(vbase + d * 512));
 
         f32x4 s[2];
 #pragma unroll

@@ -15,11 +15,12 @@ __global__ __launch_bounds__(64)
 void attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
                          T* __restrict__ out, const int* __restrict__ positions,
                          const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
-                         int max_blocks, int H, int G, int hd, int ps, int vis, int span, float scale) {
+                         int max_blocks, int H, int G, int hd, int ps, int vis, int span, float scale, int kv_tiled) {
     extern __shared__ float smem[];
     float* q_sh = smem;                 // [hd]
     float* p_sh = smem + hd;            // [64]
-    long long* row_sh = (long long*)(p_sh + 64);   // [64] element offset of each key's value column, -1 = none
+    long long* row_sh = (long long*)(p_sh + 64);   // [64] first element of the kv head's part of each key's page, -1 = none
+    int* off_sh = (int*)(row_sh + 64);             // [64] the key's offset in its page
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int g = h / (H / G);
     const int p = positions[t];
@@ -44,10 +45,10 @@ void attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
                 s = NAN;   // a page that was given back is asked for: poison the result
             } else {
                 const long long pg = (long long)page * G + g;
-                row = pg * hd * ps + (j % ps);            // value pages are [page][kv head][hd][offset]
-                const T* kr = k_pages + (pg * ps + (j % ps)) * hd;
+                row = pg * hd * ps;
+                const T* kr = k_pages + row;
                 float acc = 0.f;
-                for (int c = 0; c < hd; ++c) acc = fmaf(q_sh[c], to_f32<T>(kr[c]), acc);
+                for (int c = 0; c < hd; ++c) acc = fmaf(q_sh[c], to_f32<T>(kr[sp_k_index(j % ps, c, hd, kv_tiled)]), acc);
                 s = acc * scale;
             }
         }
@@ -59,6 +60,7 @@ void attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
         __syncthreads();
         p_sh[lane] = pj;
         row_sh[lane] = row;
+        off_sh[lane] = j % ps;
         __syncthreads();
         const int n_valid = (p - j0 + 1) < 64 ? (p - j0 + 1) : 64;
 #pragma unroll
@@ -68,7 +70,7 @@ void attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
                 float acc = o[u] * alpha;
                 for (int jj = 0; jj < n_valid; ++jj) {
                     const long long r = row_sh[jj];
-                    const float vv = r >= 0 ? to_f32<T>(v_pages[r + (long long)c * ps]) : 0.f;
+                    const float vv = r >= 0 ? to_f32<T>(v_pages[r + (long long)sp_v_index(c, off_sh[jj], hd, ps, kv_tiled)]) : 0.f;
                     acc = fmaf(p_sh[jj], vv, acc);
                 }
                 o[u] = acc;
@@ -87,21 +89,23 @@ void attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
 extern "C" int spite_attn_generic(const void* q, const void* k_pages, const void* v_pages, void* out, int dtype,
                                   const int* positions, const int* seq_of_token, const int* block_table,
                                   int max_blocks, int T, int H, int G, int hd, int page_size, int vis, int span,
-                                  float scale, hipStream_t st) {
+                                  float scale, int kv_tiled, hipStream_t st) {
     SP_REQUIRE(T >= 0 && H > 0 && G > 0 && H % G == 0, "attention: %d query heads over %d kv heads", H, G);
     SP_REQUIRE(hd > 0 && hd <= 64 * ATT_MAX_D, "attention: head size %d, at most %d", hd, 64 * ATT_MAX_D);
     SP_REQUIRE(page_size > 0 && max_blocks > 0, "attention: bad page size %d or table width %d", page_size, max_blocks);
     SP_REQUIRE(vis == SP_VIS_FULL || span > 0, "attention: chunk or window of %d", span);
     SP_REQUIRE(H <= 65535, "attention: too many heads");
+    SP_REQUIRE(!kv_tiled || (dtype == SP_BF16 && hd % 32 == 0 && page_size % 32 == 0),
+               "attention: pages in operand order are bfloat16 with head size %d and page size %d multiples of 32", hd, page_size);
     if (T == 0) return 0;
     dim3 grid(T, H);
-    const size_t sh = (size_t)(hd + 64) * sizeof(float) + 64 * sizeof(long long) + 8;
+    const size_t sh = (size_t)(hd + 64) * sizeof(float) + 64 * sizeof(long long) + 64 * sizeof(int) + 8;
     if (dtype == SP_F32)
         attn_generic_kernel<float><<<grid, 64, sh, st>>>((const float*)q, (const float*)k_pages, (const float*)v_pages,
-            (float*)out, positions, seq_of_token, block_table, max_blocks, H, G, hd, page_size, vis, span, scale);
+            (float*)out, positions, seq_of_token, block_table, max_blocks, H, G, hd, page_size, vis, span, scale, kv_tiled);
     else if (dtype == SP_BF16)
         attn_generic_kernel<bf16><<<grid, 64, sh, st>>>((const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages,
-            (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, hd, page_size, vis, span, scale);
+            (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, hd, page_size, vis, span, scale, kv_tiled);
     else return sp_fail("attention: unknown dtype %d", dtype);
     SP_LAUNCH_CHECK("attn_generic");
     return 0;

@@ -17,17 +17,18 @@
 // a wave sees whole skip the tests, blocks that none sees are skipped.
 //
 // Order of keys.  The score product leaves lane (n, qd) with rows qd*4 .. qd*4+3 of each
-// 16-row tile; the second product wants 8 consecutive k indices per lane.  K rows are
-// therefore stored in LDS permuted, so that rows qd*4+i of the two tiles of a 32-key half
-// are the keys qd*8 + i and qd*8 + 4 + i: a lane's eight probabilities of a half belong to
-// eight consecutive keys, and its V^T operand is one 16-byte read.
+// 16-row tile; the second product wants 8 consecutive k indices per lane.  The rows qd*4+i of
+// the two tiles of a 32-key half are therefore the keys qd*8 + i and qd*8 + 4 + i: a lane's
+// eight probabilities of a half belong to eight consecutive keys, and its V^T operand is one
+// 16-byte read.  The pages hold keys and values in exactly these operand tiles (common.h), one
+// kilobyte each in lane order; a block is copied to LDS as it lies, and a wave's operand read
+// is 16 bytes per lane in a row, free of bank conflicts.
 // Scores, running maximum and sum, and the output are fp32; P is rounded to bf16 only as an
 // MFMA operand.
 #include "common.h"
 
 #define PF_COLS 256        // columns (query, head) per workgroup
 #define PF_KEYS 64         // keys per block
-#define PF_VLD (PF_KEYS + 8)
 
 template <int HD>
 __global__ __launch_bounds__(512)
@@ -37,12 +38,13 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
                          const int* __restrict__ block_table, int max_blocks, int tile_q,
                          int H, int G, int ps, int vis, int span, float scale_log2e) {
     constexpr int NC = HD / 32, ND = HD / 16;
-    constexpr int KLD = HD + 8;                      // padded K row in LDS (elements)
     constexpr int KCH = PF_KEYS * HD / 8 / 512;      // 16-byte chunks of the K block per thread
     constexpr int VCH = HD * PF_KEYS / 8 / 512;      // and of the V^T block
+    constexpr int KHALF = 2 * NC * 64;               // chunks of one 32-key half of a K block
+    constexpr int VHALF = ND * 64;                   // and of a V^T block
     extern __shared__ __attribute__((aligned(16))) bf16 sm[];
-    bf16* Ks = sm;                                   // [2][64 * KLD]
-    bf16* Vs = sm + 2 * PF_KEYS * KLD;               // [2][HD * PF_VLD]
+    bf16* Ks = sm;                                   // [2][half][tile tt][chunk cc][512]
+    bf16* Vs = sm + 2 * PF_KEYS * HD;                // [2][half][tile d][512]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, qd = lane >> 4;
@@ -107,40 +109,28 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
     auto stage_load = [&](int kb) {
         const int key0 = kb * PF_KEYS;
         const int pg0 = page_of(key0), pg1 = page_of(key0 + 32);
-        const int off0 = key0 % ps, off1 = (key0 + 32) % ps;
+        const int blk0 = (key0 % ps) >> 5, blk1 = ((key0 + 32) % ps) >> 5;     // the 32-key blocks inside their pages
         // pages that are absent are read as page 0: their keys are masked, or poisoned below
-        const size_t base0 = (size_t)(pg0 < 0 ? 0 : pg0) * G + g, base1 = (size_t)(pg1 < 0 ? 0 : pg1) * G + g;
+        const size_t slab0 = ((size_t)(pg0 < 0 ? 0 : pg0) * G + g) * (size_t)ps * HD;
+        const size_t slab1 = ((size_t)(pg1 < 0 ? 0 : pg1) * G + g) * (size_t)ps * HD;
 #pragma unroll
         for (int i = 0; i < KCH; ++i) {
             const int c = tid + 512 * i;
-            const int key = c / (HD / 8), part = c % (HD / 8);
-            const size_t row = key < 32 ? base0 * ps + off0 + key : base1 * ps + off1 + (key - 32);
-            kreg[i] = *(const bf16x8*)(k_pages + row * HD + part * 8);
+            const size_t at = c < KHALF ? slab0 + ((size_t)blk0 * KHALF + c) * 8 : slab1 + ((size_t)blk1 * KHALF + (c - KHALF)) * 8;
+            kreg[i] = *(const bf16x8*)(k_pages + at);
         }
 #pragma unroll
         for (int i = 0; i < VCH; ++i) {
             const int c = tid + 512 * i;
-            const int d = c / 8, kc = c % 8;
-            const size_t at = kc < 4 ? (base0 * HD + d) * ps + off0 + kc * 8 : (base1 * HD + d) * ps + off1 + (kc - 4) * 8;
+            const size_t at = c < VHALF ? slab0 + ((size_t)blk0 * VHALF + c) * 8 : slab1 + ((size_t)blk1 * VHALF + (c - VHALF)) * 8;
             vreg[i] = *(const bf16x8*)(v_pages + at);
         }
     };
     auto stage_store = [&](int buf) {
-        bf16* kb_ = Ks + buf * PF_KEYS * KLD;
-        bf16* vb_ = Vs + buf * HD * PF_VLD;
 #pragma unroll
-        for (int i = 0; i < KCH; ++i) {
-            const int c = tid + 512 * i;
-            const int key = c / (HD / 8), part = c % (HD / 8);
-            const int w = key & 31;
-            const int row = (key & 32) + ((w >> 2) & 1) * 16 + (w >> 3) * 4 + (w & 3);
-            *(bf16x8*)(kb_ + row * KLD + part * 8) = kreg[i];
-        }
+        for (int i = 0; i < KCH; ++i) *(bf16x8*)(Ks + buf * PF_KEYS * HD + (tid + 512 * i) * 8) = kreg[i];
 #pragma unroll
-        for (int i = 0; i < VCH; ++i) {
-            const int c = tid + 512 * i;
-            *(bf16x8*)(vb_ + (c / 8) * PF_VLD + (c % 8) * 8) = vreg[i];
-        }
+        for (int i = 0; i < VCH; ++i) *(bf16x8*)(Vs + buf * HD * PF_KEYS + (tid + 512 * i) * 8) = vreg[i];
     };
 
     // ---- one block of 64 keys out of LDS
@@ -149,14 +139,14 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
         if (key0 > pq_max || key0 + PF_KEYS - 1 < lo_min) return;     // nothing here for this wave
         const bool whole = key0 >= lo_max && key0 + PF_KEYS - 1 <= pq_min;
         const bool absent0 = page_of(key0) < 0, absent1 = page_of(key0 + 32) < 0;
-        const bf16* kb_ = Ks + buf * PF_KEYS * KLD;
-        const bf16* vb_ = Vs + buf * HD * PF_VLD;
+        const bf16* kb_ = Ks + buf * PF_KEYS * HD + lane * 8;
+        const bf16* vb_ = Vs + buf * HD * PF_KEYS + lane * 8;
         f32x4 s[2][4];
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) {
             bf16x8 kf[NC];
 #pragma unroll
-            for (int cc = 0; cc < NC; ++cc) kf[cc] = *(const bf16x8*)(kb_ + (tt * 16 + n) * KLD + cc * 32 + qd * 8);
+            for (int cc = 0; cc < NC; ++cc) kf[cc] = *(const bf16x8*)(kb_ + (tt * NC + cc) * 512);
 #pragma unroll
             for (int c = 0; c < 2; ++c) {
                 s[c][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -215,7 +205,7 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
             for (int c = 0; c < 2; ++c) o[c][d] = o[c][d] * alpha[c];
 #pragma unroll
             for (int hh = 0; hh < 2; ++hh) {
-                const bf16x8 vf = *(const bf16x8*)(vb_ + (d * 16 + n) * PF_VLD + hh * 32 + qd * 8);
+                const bf16x8 vf = *(const bf16x8*)(vb_ + (hh * ND + d) * 512);
 #pragma unroll
                 for (int c = 0; c < 2; ++c)
                     o[c][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[c][hh], o[c][d], 0, 0, 0);
@@ -273,7 +263,7 @@ extern "C" int spite_attn_prefill(const void* q, const void* k_pages, const void
     SP_REQUIRE(n_tiles <= 0x7fffffffL, "attn_prefill: too many tiles");
     const float sl = scale * 1.4426950408889634f;
     dim3 grid((unsigned)n_tiles, G);
-    const size_t sh = (size_t)2 * (PF_KEYS * (hd + 8) + hd * PF_VLD) * sizeof(bf16);
+    const size_t sh = (size_t)2 * 2 * PF_KEYS * hd * sizeof(bf16);
     static bool allowed[2] = {false, false};     // the kernels ask for more LDS than the default limit
     if (hd == 128) {
         if (!allowed[0]) {

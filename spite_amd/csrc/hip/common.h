@@ -32,6 +32,28 @@ __device__ __forceinline__ int sp_first_visible(int p, int vis, int span) {
     return 0;
 }
 
+// ---- layouts of one kv head's part of a cache page.
+// Row-major: keys [page_size][hd], values transposed [hd][page_size].
+// Operand order (bf16, hd % 32 == 0, page_size % 32 == 0): the MFMA attention kernels' operand
+// tiles, each one kilobyte in lane order, so that a wave's load is a run of whole cache lines.
+//   keys:   blocks of 32 keys; block b holds two tiles tt of 16 rows, row r of tile tt being the
+//           key (r/4)*8 + tt*4 + r%4 of the block, each tile cut into hd/32 chunks cc of 32
+//           elements: tile (b, tt, cc) at ((b*2 + tt) * hd/32 + cc) * 512, inside it element
+//           8q+e of row r at (q*16 + r)*8 + e.
+//   values: block b, 16 head elements dt*16 .. dt*16+15 as rows, the block's 32 keys as k:
+//           tile (b, dt) at (b * hd/16 + dt) * 512, inside it key 8q+e of row r at (q*16 + r)*8 + e.
+__device__ __forceinline__ size_t sp_k_index(int off, int c, int hd, bool tiled) {
+    if (!tiled) return (size_t)off * hd + c;
+    const int b = off >> 5, w = off & 31;
+    const int r = ((w >> 3) << 2) | (w & 3), tt = (w >> 2) & 1;
+    return ((size_t)(b * 2 + tt) * (hd >> 5) + (c >> 5)) * 512 + (size_t)(((((c & 31) >> 3) << 4) + r) << 3) + (c & 7);
+}
+__device__ __forceinline__ size_t sp_v_index(int c, int off, int hd, int ps, bool tiled) {
+    if (!tiled) return (size_t)c * ps + off;
+    const int b = off >> 5, w = off & 31;
+    return ((size_t)b * (hd >> 4) + (c >> 4)) * 512 + (size_t)((((w >> 3) << 4) + (c & 15)) << 3) + (w & 7);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);

@@ -185,7 +185,7 @@ void rope_kvwrite_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
                          const int* __restrict__ positions, const int* __restrict__ slot_map,
                          const float* __restrict__ inv_freq, int H, int G, int hd, int ps,
                          int use_rope, int adjacent, int use_norm, float norm_eps,
-                         int use_temp, int floor_scale, float attn_scale, int n_heads, int hpw) {
+                         int use_temp, int floor_scale, float attn_scale, int n_heads, int hpw, int kv_tiled) {
     const int t = blockIdx.x;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int half = hd >> 1;
@@ -210,18 +210,22 @@ void rope_kvwrite_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
         const bool is_q = hh < H;
         const bool is_v = hh >= H + G;
         T* dst;
+        int off = 0;
+        const bool tiled_k = !is_q && kv_tiled;      // the key's elements go to their places in the operand tiles
         if (is_q) {
             dst = q_out + ((size_t)t * H + hh) * hd;
         } else {
             if (slot < 0) continue;
             const int g = is_v ? hh - H - G : hh - H;
-            const size_t page = slot / ps, off = slot % ps;
+            const size_t page = slot / ps;
+            off = slot % ps;
             if (is_v) {
-                T* col = v_pages + (page * G + g) * hd * ps + off;
-                for (int c = lane; c < hd; c += 64) col[(size_t)c * ps] = src[c];
+                T* slab = v_pages + (page * G + g) * hd * ps;
+                for (int c = lane; c < hd; c += 64) slab[sp_v_index(c, off, hd, ps, kv_tiled)] = src[c];
                 continue;
             }
-            dst = k_pages + ((page * G + g) * ps + off) * hd;
+            dst = k_pages + (page * G + g) * (size_t)ps * hd;
+            if (!kv_tiled) dst += (size_t)off * hd;
         }
         float x0[SP_MAX_PAIRS], x1[SP_MAX_PAIRS];
         float ss = 0.f;
@@ -253,8 +257,8 @@ void rope_kvwrite_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
             if (i < half) {
                 const int i0 = adjacent ? 2 * i : i;
                 const int i1 = adjacent ? 2 * i + 1 : i + half;
-                dst[i0] = from_f32<T>(x0[u] * scale);
-                dst[i1] = from_f32<T>(x1[u] * scale);
+                dst[tiled_k ? sp_k_index(off, i0, hd, true) : (size_t)i0] = from_f32<T>(x0[u] * scale);
+                dst[tiled_k ? sp_k_index(off, i1, hd, true) : (size_t)i1] = from_f32<T>(x1[u] * scale);
             }
         }
     }
@@ -264,7 +268,7 @@ extern "C" int spite_rope_kvwrite(const void* qkv, void* q_out, void* k_pages, v
                                   const int* positions, const int* slot_map, const float* inv_freq,
                                   int T, int H, int G, int hd, int page_size, int use_rope, int adjacent,
                                   int use_norm, float norm_eps, int use_temp, int floor_scale,
-                                  float attn_scale, int write_kv, hipStream_t st) {
+                                  float attn_scale, int write_kv, int kv_tiled, hipStream_t st) {
     SP_REQUIRE(T >= 0 && H > 0 && G > 0 && hd > 0 && page_size > 0, "rope_kvwrite: bad sizes");
     SP_REQUIRE(hd % 2 == 0 && hd <= 128 * SP_MAX_PAIRS, "rope_kvwrite: head size %d must be even and <= %d",
                hd, 128 * SP_MAX_PAIRS);
@@ -272,6 +276,8 @@ extern "C" int spite_rope_kvwrite(const void* qkv, void* q_out, void* k_pages, v
     SP_REQUIRE(!use_rope || inv_freq, "rope_kvwrite: rotation needs a frequency table");
     SP_REQUIRE(H + 2 * G <= 65535, "rope_kvwrite: too many heads");
     SP_REQUIRE(!write_kv || slot_map, "rope_kvwrite: writing the cache needs the rows' slots");
+    SP_REQUIRE(!kv_tiled || (dtype == SP_BF16 && hd % 32 == 0 && page_size % 32 == 0),
+               "rope_kvwrite: pages in operand order are bfloat16 with head size %d and page size %d multiples of 32", hd, page_size);
     if (T == 0) return 0;
     const int n_heads = write_kv ? H + 2 * G : H;
     const int hpw = T >= 256 ? 4 : 1;            // many tokens: fewer, longer workgroups
@@ -279,11 +285,11 @@ extern "C" int spite_rope_kvwrite(const void* qkv, void* q_out, void* k_pages, v
     if (dtype == SP_F32)
         rope_kvwrite_kernel<float><<<grid, 256, 0, st>>>((const float*)qkv, (float*)q_out, (float*)k_pages,
             (float*)v_pages, positions, slot_map, inv_freq, H, G, hd, page_size, use_rope, adjacent, use_norm,
-            norm_eps, use_temp, floor_scale, attn_scale, n_heads, hpw);
+            norm_eps, use_temp, floor_scale, attn_scale, n_heads, hpw, kv_tiled);
     else if (dtype == SP_BF16)
         rope_kvwrite_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)qkv, (bf16*)q_out, (bf16*)k_pages,
             (bf16*)v_pages, positions, slot_map, inv_freq, H, G, hd, page_size, use_rope, adjacent, use_norm,
-            norm_eps, use_temp, floor_scale, attn_scale, n_heads, hpw);
+            norm_eps, use_temp, floor_scale, attn_scale, n_heads, hpw, kv_tiled);
     else return sp_fail("rope_kvwrite: unknown dtype %d", dtype);
     SP_LAUNCH_CHECK("rope_kvwrite");
     return 0;

@@ -35,12 +35,12 @@ def lib():
         sigs = {
             "spite_embed": [P, P, I, P, I, I, I, P],
             "spite_add_rmsnorm": [P, P, P, P, P, I, P, P, I, I, F, I, P, P, I, P],
-            "spite_rope_kvwrite": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, I, I, F, I, P],
+            "spite_rope_kvwrite": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, I, I, F, I, I, P],
             "spite_router_top1": [P, P, P, P, P, I, I, I, P],
             "spite_moe_plan": [P, P, P, P, P, P, P, I, I, I, P],
             "spite_convert": [P, I, P, I, c_size_t, P],
             "spite_gemm_generic": [P, I, P, L, I, P, I, I, I, I, I, P, I, P, P, P, I, P],
-            "spite_attn_generic": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, P],
+            "spite_attn_generic": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, I, P],
             "spite_sample_rows": [P, I, I, I, P, P, P, P],
             "spite_gemm_skinny": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, I, I, P],
             "spite_attn_decode": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, P],
@@ -140,7 +140,8 @@ def add_rmsnorm(h, w, eps, out=None, out32=None, d1=None, d2=None, rows=None, n_
 
 
 def rope_kvwrite(qkv, q_out, k_pages, v_pages, positions, slot_map, inv_freq, H, G, hd, page_size, *,
-                 use_rope, adjacent, use_norm, norm_eps, use_temp, floor_scale, attn_scale, write_kv=True):
+                 use_rope, adjacent, use_norm, norm_eps, use_temp, floor_scale, attn_scale, write_kv=True,
+                 kv_tiled=False):
     """Rotation, weightless qk-norm and temperature of the fused projection's rows; keys and
     values go to their cache rows.  qkv [T,(H+2G)*hd]; q_out [T,H*hd]; key pages
     [n_pages, G, page_size, hd], value pages [n_pages, G, hd, page_size]."""
@@ -161,7 +162,7 @@ def rope_kvwrite(qkv, q_out, k_pages, v_pages, positions, slot_map, inv_freq, H,
         _ptr(v_pages, "v_pages", dt, not write_kv), dtype_code(dt), _ptr(positions, "positions", torch.int32),
         _ptr(slot_map, "slot_map", torch.int32, not write_kv), _ptr(inv_freq, "inv_freq", torch.float32, not use_rope),
         T, H, G, hd, page_size, int(use_rope), int(adjacent), int(use_norm), float(norm_eps), int(use_temp),
-        int(floor_scale), float(attn_scale), int(write_kv), _stream()), "rope_kvwrite")
+        int(floor_scale), float(attn_scale), int(write_kv), int(bool(kv_tiled)), _stream()), "rope_kvwrite")
 
 
 def router_top1(x32, w_router, expert, weight, logits_out=None):
@@ -231,9 +232,10 @@ def gemm_generic(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_s
 
 
 def attn_generic(q, k_pages, v_pages, out, positions, seq_of_token, block_table, T, H, G, hd, page_size,
-                 vis, span, scale):
+                 vis, span, scale, kv_tiled=False):
     """Attention over the paged cache, any mix of portions and single tokens.  q/out
-    [T,H*hd]; block_table int32 [n_seqs, max_blocks]."""
+    [T,H*hd]; block_table int32 [n_seqs, max_blocks].  ``kv_tiled``: the pages are in operand
+    order (``kv_operand_order``)."""
     if q.numel() < T * H * hd or out.numel() < T * H * hd:
         raise KernelError("attention: q or out too small")
     _check_pages(k_pages, v_pages, G, page_size, hd, "attention")
@@ -244,7 +246,7 @@ def attn_generic(q, k_pages, v_pages, out, positions, seq_of_token, block_table,
         _ptr(q, "q"), _ptr(k_pages, "k_pages", dt), _ptr(v_pages, "v_pages", dt), _ptr(out, "out", dt),
         dtype_code(dt), _ptr(positions, "positions", torch.int32), _ptr(seq_of_token, "seq_of_token", torch.int32),
         _ptr(block_table, "block_table", torch.int32), block_table.shape[1], T, H, G, hd, page_size,
-        VIS[vis], int(span or 0), float(scale), _stream()), "attention")
+        VIS[vis], int(span or 0), float(scale), int(bool(kv_tiled)), _stream()), "attention")
 
 
 def sample_rows(logits, temperature, uniform, out, n_rows=None):
@@ -296,6 +298,29 @@ def gemm_skinny(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_sc
         int(max_rows if max_rows is not None else M), int(variant), int(bool(tiled)), _stream()), "gemm_skinny")
 
 
+def kv_tiled_ok(dtype, hd, page_size) -> bool:
+    """Whether cache pages of this kind are kept in MFMA operand order."""
+    return dtype == torch.bfloat16 and hd % 32 == 0 and page_size % 32 == 0
+
+
+def kv_operand_order(k_pages, v_pages):
+    """Copies of row-major pages (keys [n, G, page_size, hd], values transposed [n, G, hd,
+    page_size]) in the operand order that the MFMA attention kernels read; same shapes.
+    Keys: blocks of 32 keys, two tiles of 16 rows (row r of tile tt = key (r/4)*8 + tt*4 + r%4),
+    hd/32 chunks each, a tile's [16 rows][32 elements] stored as [4 q][16 r][8 e].  Values:
+    per block of 32 keys, tiles of 16 head elements, [16 rows][32 keys] stored the same way."""
+    n, G, ps, hd = k_pages.shape
+    if ps % 32 or hd % 32:
+        raise KernelError(f"operand order needs page size {ps} and head size {hd} to be multiples of 32")
+    # key offset w = 8a + 4tt + i  ->  row r = 4a + i of tile tt; element c = 32cc + 8q + e
+    k = k_pages.reshape(n, G, ps // 32, 4, 2, 4, hd // 32, 4, 8)          # b, a, tt, i, cc, q, e
+    k = k.permute(0, 1, 2, 4, 6, 7, 3, 5, 8)                                # b, tt, cc, q, a, i, e
+    # head element c = 16dt + r, key offset = 32b + 8q + e
+    v = v_pages.reshape(n, G, hd // 16, 16, ps // 32, 4, 8)                # dt, r, b, q, e
+    v = v.permute(0, 1, 4, 2, 5, 3, 6)                                      # b, dt, q, r, e
+    return k.contiguous().view(n, G, ps, hd), v.contiguous().view(n, G, hd, ps)
+
+
 def attn_decode_workspace(T, H, hd, n_splits) -> int:
     """Bytes of scratch that attn_decode needs."""
     return T * H * n_splits * (hd + 2) * 4
@@ -304,7 +329,7 @@ def attn_decode_workspace(T, H, hd, n_splits) -> int:
 def attn_decode(q, k_pages, v_pages, out, workspace, positions, seq_of_token, block_table, T, H, G, hd,
                 page_size, vis, span, scale, n_splits):
     """Split-KV decode attention on MFMA (bf16; head sizes 64 and 128; pages of a multiple of 32
-    keys): every row of q is one query against its request's cache."""
+    keys, in operand order): every row of q is one query against its request's cache."""
     if q.dtype != torch.bfloat16:
         raise KernelError(f"attn_decode: bfloat16 only, got {q.dtype}")
     if q.numel() < T * H * hd or out.numel() < T * H * hd:
@@ -364,7 +389,8 @@ def gemm_tiled(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_sca
 
 def attn_prefill(q, k_pages, v_pages, out, positions, cu_seqlens, counts, block_table,
                  H, G, hd, page_size, vis, span, scale):
-    """Prefill attention on MFMA (bf16; head sizes 64 and 128; pages of a multiple of 32 keys).
+    """Prefill attention on MFMA (bf16; head sizes 64 and 128; pages of a multiple of 32 keys, in
+    operand order).
     ``counts``: the number of query tokens of every request of the step, on the host, in the
     order of ``cu_seqlens`` (their running sum, on the device) and of the block table's rows."""
     if q.dtype != torch.bfloat16:

@@ -68,6 +68,7 @@ class LayerCache:
     page_size: int
     write: bool                           # this call fills the cache (else it reads another layer's)
     state: Optional[torch.Tensor] = None  # [max_requests, ...]: per-request state of the layer
+    tiled: bool = False                   # pages in the MFMA attention kernels' operand order, not row-major
 
 
 @dataclass

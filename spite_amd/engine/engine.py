@@ -106,7 +106,8 @@ class StepMeta:
             return LayerCache(None, None, None, None, cache.page_size, call.write, state)
         g = cache.group_of(call.cache)
         k, v = cache.layer_pages(call.cache)
-        return LayerCache(k, v, self.slot_maps[g], self.tables[g], cache.page_size, call.write, state)
+        return LayerCache(k, v, self.slot_maps[g], self.tables[g], cache.page_size, call.write, state,
+                          cache.kv_tiled(call.cache))
 
 
 class Engine:

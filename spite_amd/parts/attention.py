@@ -76,10 +76,10 @@ class Attention(Mixer):
                             H, G, hd, cache.page_size, use_rope=ka["use_rope"], adjacent=ka["adjacent"],
                             use_norm=self.qk_norm, norm_eps=self.qk_norm_eps, use_temp=temp is not None,
                             floor_scale=temp[0] if temp else 1, attn_scale=temp[1] if temp else 0.0,
-                            write_kv=cache.write)
+                            write_kv=cache.write, kv_tiled=cache.tiled)
         o = ws.take((T, H * hd), x.dtype)
-        if (ctx.decode_only and x.dtype == torch.bfloat16 and hd in (64, 128) and cache.page_size % 32 == 0
-                and H // G <= 16):
+        # the MFMA kernels read pages in operand order (bfloat16, sizes in multiples of 32)
+        if ctx.decode_only and cache.tiled and hd in (64, 128) and H // G <= 16:
             # split the keys so that about five hundred workgroups run (measured: more splits only
             # add partial results to combine), each wave with at least one block of keys; the
             # bound on the keys is the block table's width, so the launch is the same for every
@@ -93,13 +93,13 @@ class Attention(Mixer):
             hipops.attn_decode(q, cache.k_pages, cache.v_pages, o, scratch, ctx.positions, ctx.seq_of_token,
                                cache.block_table, T, H, G, hd, cache.page_size, self.visibility, self.span,
                                self.scale, n_splits)
-        elif x.dtype == torch.bfloat16 and hd in (64, 128) and cache.page_size % 32 == 0:
+        elif cache.tiled and hd in (64, 128):
             hipops.attn_prefill(q, cache.k_pages, cache.v_pages, o, ctx.positions, ctx.cu_seqlens, ctx.host.counts,
                                 cache.block_table, H, G, hd, cache.page_size, self.visibility, self.span, self.scale)
         else:
             hipops.attn_generic(q, cache.k_pages, cache.v_pages, o, ctx.positions, ctx.seq_of_token,
                                 cache.block_table, T, H, G, hd, cache.page_size, self.visibility, self.span,
-                                self.scale)
+                                self.scale, kv_tiled=cache.tiled)
         out = ws.take((T, self.d), torch.float32)
         linear(o, self.wo, out)
         return out

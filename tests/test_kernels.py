@@ -99,6 +99,17 @@ def test_rope_kvwrite(dtype, H, G, hd, adjacent, norm, temp, T):
         page, off = int(slots[t]) // ps, int(slots[t]) % ps
         assert (kp[page, :, off].double().cpu() - rk[t]).abs().max() < tol
         assert torch.equal(vp[page, :, :, off].cpu().double(), vv[t])
+    if ops().kv_tiled_ok(dtype, hd, 32):       # the same rows into pages of 32 in operand order
+        kp32 = torch.zeros(n_pages, G, 32, hd, dtype=dtype, device=DEV)
+        vp32 = torch.zeros(n_pages, G, hd, 32, dtype=dtype, device=DEV)
+        kpt, vpt, q2 = torch.zeros_like(kp32), torch.zeros_like(vp32), torch.empty_like(q)
+        slots32 = (slots // ps) * 32 + ((slots % ps) * 9 + (slots // ps)) % 32        # spread over the page's offsets
+        for tiled, (a, b) in ((False, (kp32, vp32)), (True, (kpt, vpt))):
+            ops().rope_kvwrite(qkv, q2, a, b, pos, slots32, inv, H, G, hd, 32, use_rope=True, adjacent=adjacent,
+                               use_norm=norm, norm_eps=1e-5, use_temp=temp, floor_scale=4, attn_scale=0.1, kv_tiled=tiled)
+            assert torch.equal(q2, q)
+        want_k, want_v = ops().kv_operand_order(kp32, vp32)
+        assert float(kp32.abs().sum()) > 0 and torch.equal(kpt, want_k) and torch.equal(vpt, want_v)
     written = {(int(s) // ps, int(s) % ps) for s in slots.cpu()}
     for p in range(n_pages):
         for o in range(ps):
@@ -294,8 +305,15 @@ def run_attention(kind, dtype, H, G, hd, ps, lens, queries, vis, span, n_splits=
     out = torch.zeros(T, H * hd, dtype=dtype, device=DEV)
     q_dev, kp, vp, bt = qs.reshape(T, H * hd).to(DEV), kv.kp.to(DEV), kv.vp.to(DEV), kv.bt.to(DEV)
     scale = 1.0 / math.sqrt(hd)
+    if kind != "generic":                        # the MFMA kernels read pages in operand order
+        kp, vp = ops().kv_operand_order(kp, vp)
     if kind == "generic":
         ops().attn_generic(q_dev, kp, vp, out, positions, seq, bt, T, H, G, hd, ps, vis, span, scale)
+        if ops().kv_tiled_ok(dtype, hd, ps):     # and the plain kernel reads them too, with the same bits
+            again = torch.zeros_like(out)
+            kpt, vpt = ops().kv_operand_order(kp, vp)
+            ops().attn_generic(q_dev, kpt, vpt, again, positions, seq, bt, T, H, G, hd, ps, vis, span, scale, kv_tiled=True)
+            assert torch.equal(out, again)
     elif kind == "prefill":                      # runs of queries of one request are the portions
         runs = []
         for s, _ in queries:
@@ -390,7 +408,7 @@ def test_attn_prefill(case):
         cu.append(cu[-1] + count)
     bt = torch.stack([kv.bt[s] for s, _, _ in portions]).to(DEV)
     out = torch.zeros(T, H * hd, dtype=dtype, device=DEV)
-    ops().attn_prefill(qs.reshape(T, H * hd).to(DEV), kv.kp.to(DEV), kv.vp.to(DEV), out, positions,
+    ops().attn_prefill(qs.reshape(T, H * hd).to(DEV), *ops().kv_operand_order(kv.kp.to(DEV), kv.vp.to(DEV)), out, positions,
                        torch.tensor(cu, dtype=torch.int32, device=DEV), [count for _, _, count in portions], bt,
                        H, G, hd, ps, vis, span, 1.0 / math.sqrt(hd))
     got = out.double().cpu().view(T, H, hd)
