@@ -1,6 +1,9 @@
 // Decode attention over the paged cache on MFMA: one query token per request, the visible
 // keys of a request split over workgroups ("split-KV"), partial (max, sum, output) per split
-// in fp32, then a small kernel that combines the splits.
+// in fp32, then a small kernel that combines the splits.  (Letting the workgroup that
+// finishes last combine them was measured four times slower: making the partial results
+// visible across the chip's L2 caches costs more than the second launch.)  With one split the
+// output is written at once.
 //
 // A workgroup serves one token, one kv head and one split; the H/G query heads that share
 // the kv head are the 16 columns of the MFMA tiles (unused columns are zero), so K and V are
@@ -23,7 +26,7 @@
 template <int HD>
 __global__ __launch_bounds__(256)
 void attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages,
-                        const bf16* __restrict__ v_pages, float* __restrict__ part,
+                        const bf16* __restrict__ v_pages, float* __restrict__ part, bf16* __restrict__ out,
                         const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                         const int* __restrict__ block_table, int max_blocks, int H, int G, int ps, int vis,
                         int span, float scale_log2e, int n_splits) {
@@ -127,6 +130,24 @@ void attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_p
         for (int i = 0; i < 4; ++i) mine[d * 16 + qd * 4 + i] = o[d][i];
     if (qd == 0) { mine[HD] = m_run; mine[HD + 1] = l_run; }
     __syncthreads();
+    if (n_splits == 1) {                 // nothing to combine: the four waves' sums are the result
+        for (int idx = threadIdx.x; idx < QH * HD; idx += 256) {
+            const int hn = idx / HD, c = idx % HD;
+            float M = -INFINITY;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) M = fmaxf(M, sm[((size_t)w * 16 + hn) * ROW + HD]);
+            float acc = 0.f, L = 0.f;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const float mw = sm[((size_t)w * 16 + hn) * ROW + HD];
+                const float f = (mw == -INFINITY) ? 0.f : exp2f(mw - M);
+                acc += f * sm[((size_t)w * 16 + hn) * ROW + c];
+                L += f * sm[((size_t)w * 16 + hn) * ROW + HD + 1];
+            }
+            out[((size_t)t * H + g * QH + hn) * HD + c] = (bf16)(acc * (1.0f / fmaxf(L, 1e-30f)));
+        }
+        return;
+    }
     for (int idx = threadIdx.x; idx < QH * ROW; idx += 256) {
         const int hn = idx / ROW, c = idx % ROW;
         float M = -INFINITY;
@@ -206,14 +227,16 @@ extern "C" int spite_attn_decode(const void* q, const void* k_pages, const void*
     const size_t sh = (size_t)4 * 16 * (hd + 2) * sizeof(float);
     if (hd == 128) {
         attn_decode_kernel<128><<<grid, 256, sh, st>>>((const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages,
-            (float*)workspace, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, n_splits);
+            (float*)workspace, (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, n_splits);
         SP_LAUNCH_CHECK("attn_decode");
-        attn_decode_combine_kernel<128><<<dim3(T, H), 128, 0, st>>>((const float*)workspace, (bf16*)out, H, n_splits);
+        if (n_splits > 1)
+            attn_decode_combine_kernel<128><<<dim3(T, H), 128, 0, st>>>((const float*)workspace, (bf16*)out, H, n_splits);
     } else {
         attn_decode_kernel<64><<<grid, 256, sh, st>>>((const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages,
-            (float*)workspace, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, n_splits);
+            (float*)workspace, (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, n_splits);
         SP_LAUNCH_CHECK("attn_decode");
-        attn_decode_combine_kernel<64><<<dim3(T, H), 64, 0, st>>>((const float*)workspace, (bf16*)out, H, n_splits);
+        if (n_splits > 1)
+            attn_decode_combine_kernel<64><<<dim3(T, H), 64, 0, st>>>((const float*)workspace, (bf16*)out, H, n_splits);
     }
     SP_LAUNCH_CHECK("attn_decode_combine");
     return 0;

@@ -150,6 +150,7 @@ class Engine:
             tokens = cache_tokens if cache_tokens is not None else self.max_requests * 4096
             num_pages = max(1, -(-int(tokens) // self.page_size))
         self.cache = PagedCache(needs, self.page_size, num_pages, self.max_requests, self.env.dtype, self.device)
+        self._folder = None
         if tensors is not None:
             self._load_from_dict(tensors, ckpt_dtype)
         elif random_weights:
@@ -158,6 +159,7 @@ class Engine:
             if not isinstance(model, str) or not os.path.isdir(model):
                 raise EngineError("without random_weights the model must be a folder with model.safetensors")
             load_weights(self.model, model, ckpt_dtype)
+            self._folder = model
         torch.cuda.empty_cache()
         self._arenas = [Workspace(self.device), Workspace(self.device)]
         self._step_ws = Workspace(self.device)
@@ -212,6 +214,25 @@ class Engine:
             owner.load(ts)
             ts.clear()
         self.model.finish_loading()
+
+    def tensor_names(self):
+        """Checkpoint names of the model's tensors, in the order of the layers."""
+        return [f for f, _, _, _ in self.model.tensor_plan()]
+
+    def get_tensor(self, name: str) -> torch.Tensor:
+        """A tensor of the model folder by its checkpoint name, as stored (on the host).  The
+        parts keep their own layouts of it on the GPU (fused, transposed, in operand order);
+        this reads the file."""
+        if self._folder is None:
+            raise EngineError("get_tensor reads the model folder; this engine was built from tensors in memory "
+                              "(write a folder with `spite random-model` to read them back)")
+        from ..weights.safetensors_io import Checkpoint
+        from ..weights.loader import _strip
+        ckpt = Checkpoint(self._folder)
+        for stored in ckpt.names():
+            if _strip(stored) == name or stored == name:
+                return ckpt.tensor(stored)
+        raise KeyError(f"{name!r} is not a tensor of {self._folder}")
 
     # ------------------------------------------------------------------ metadata transport
     def _pinned(self, n: int) -> np.ndarray:

@@ -160,3 +160,26 @@ def test_random_weights_mode_of_the_engine(models):
     b = Engine(cfg, dtype="bfloat16", random_weights=True, seed=4, page_size=32, cache_tokens=256, max_requests=2)
     p = H.random_tokens(cfg["vocab_size"], 12, 2)
     assert a.generate([p], max_tokens=5) == b.generate([p], max_tokens=5)
+
+
+def test_tensors_and_cache_can_be_looked_at(models):
+    from spite_amd import Engine
+    from spite_amd.engine.engine import EngineError, StepEntry
+    d, w, cfg = models["A"]
+    eng = engine(d)
+    names = eng.tensor_names()
+    assert "lm_head.weight" in names and "model.layers.1.feed_forward.router.weight" in names
+    assert torch.equal(eng.get_tensor("model.layers.0.self_attn.q_proj.weight"), w["model.layers.0.self_attn.q_proj.weight"])
+    with pytest.raises(KeyError):
+        eng.get_tensor("no.such.tensor")
+    with pytest.raises(EngineError, match="in memory"):
+        Engine(cfg, dtype="float32", random_weights=True, page_size=16, cache_tokens=64, max_requests=1).get_tensor("lm_head.weight")
+    # pages: 40 positions take three pages of 16 in the full group; the chunked group (chunks of 32) keeps one
+    slot = eng.admit()
+    free = [eng.cache.free_pages(g) for g in range(eng.cache.n_groups())]
+    eng.step([StepEntry(slot, H.random_tokens(cfg["vocab_size"], 40, 1), [39])])
+    held = [free[g] - eng.cache.free_pages(g) for g in range(eng.cache.n_groups())]
+    assert sorted(held) == [1, 3]
+    assert sorted(sum(p >= 0 for p in eng.cache.block_table(slot, g)) for g in range(eng.cache.n_groups())) == [1, 3]
+    eng.release(slot)
+    assert [eng.cache.free_pages(g) for g in range(eng.cache.n_groups())] == free
