@@ -1,0 +1,202 @@
+"""Other kinds of every part, defined here and registered without a change to the framework's
+files: a norm (LayerNorm with a bias), a position encoding that the fused rotation kernel does
+not know (its `transform` is called instead), and a feed-forward with its own routing (two
+experts a token, softmax over the two, the expert's *output* weighted) that walks the
+framework's grouped products with a row list of its own.  They sit in one model beside the
+built-in parts and are stepped whole, token by token, in portions and mixed."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+import helpers as H
+
+pytestmark = pytest.mark.gpu
+D, V, HEADS, KV, HD, E, FF = 32, 60, 4, 2, 8, 4, 24
+
+
+def define_parts():
+    from spite_amd.parts import Norm, FeedForward, PositionEncoding, ParamSpec, register
+    from spite_amd.parts.linear import linear, Weight
+
+    @register("norm", "toy_layernorm")
+    class LayerNorm(Norm):
+        def __init__(self, env, width, eps):
+            self.width, self.eps = width, eps
+
+        def params(self):
+            return {"weight": ParamSpec((self.width,), kind="vector", init="ones"),
+                    "bias": ParamSpec((self.width,), kind="vector", init="zeros")}
+
+        def load(self, t):
+            self.w, self.b = t["weight"], t["bias"]
+
+        def forward(self, h, out, *, d1=None, d2=None, out32=None, rows=None, write_h=True):
+            v = h
+            for d in (d1, d2):
+                if d is not None:
+                    v = v + d[:h.shape[0]]
+            if write_h and v is not h:
+                h.copy_(v)
+            if rows is not None:
+                v = v[rows.long()]
+            y = F.layer_norm(v, (self.width,), self.w, self.b, self.eps)
+            out[:y.shape[0]].copy_(y)
+            if out32 is not None:
+                out32[:y.shape[0]].copy_(y)
+
+    @register("position", "toy_scale")
+    class Scale(PositionEncoding):
+        """q and k times 1 + cos(pos * f)/2, f a tensor of the checkpoint: not a rotation."""
+        fused = False
+
+        def __init__(self, env, head_dim):
+            self.hd = head_dim
+
+        def params(self):
+            return {"freq": ParamSpec((self.hd,), kind="vector")}
+
+        def load(self, t):
+            self.freq = t["freq"]
+
+        def transform(self, qkv, positions, n_heads, n_kv_heads, head_dim):
+            T = qkv.shape[0]
+            s = 1 + 0.5 * torch.cos(positions.float()[:, None] * self.freq[None, :])
+            qk = qkv[:, :(n_heads + n_kv_heads) * head_dim].view(T, n_heads + n_kv_heads, head_dim)
+            qk.mul_(s[:, None, :].to(qkv.dtype))
+
+    @register("ffn", "toy_top2_softmax")
+    class Top2(FeedForward):
+        wants_f32_input = True
+
+        def __init__(self, env, hidden_size, intermediate_size, n_experts):
+            self.d, self.F, self.E = hidden_size, intermediate_size, n_experts
+
+        def params(self):
+            return {"router": ParamSpec((self.E, self.d), kind="vector"),
+                    "gate_up": ParamSpec((self.E, 2 * self.F, self.d)), "down": ParamSpec((self.E, self.d, self.F))}
+
+        def load(self, t):
+            self.router, self.w_gate_up, self.w_down = t["router"], Weight(t["gate_up"]), Weight(t["down"])
+
+        def forward(self, x, x32, ctx, projected=None):
+            T, E = x.shape[0], self.E
+            top = torch.topk(x32[:T] @ self.router.T, 2, dim=-1)
+            weight = torch.softmax(top.values, dim=-1).reshape(-1)          # slot 2t+k: choice k of token t
+            expert = top.indices.reshape(-1)
+            order = torch.sort(expert, stable=True).indices                  # the slots, expert by expert
+            offsets = torch.zeros(E + 1, dtype=torch.int32, device=x.device)
+            offsets[1:] = torch.cumsum(torch.bincount(expert, minlength=E), 0)
+            src = (order // 2).to(torch.int32)
+            dst = ((order % 2) * T + order // 2).to(torch.int32)             # first choices to rows [0,T), second to [T,2T)
+            scale = weight[order].float().contiguous()
+            act = ctx.ws.take((2 * T, self.F), x.dtype)
+            linear(x, self.w_gate_up, act, glu=True, offsets=offsets, n_groups=E, a_rows=src, rows=2 * T, max_rows=T)
+            y = ctx.ws.take((2 * T, self.d), torch.float32)
+            linear(act, self.w_down, y, offsets=offsets, n_groups=E, a_scale=scale, y_rows=dst, rows=2 * T, max_rows=T)
+            return (y[:T], y[T:])
+
+
+def spec():
+    from spite_amd.parts import PartSpec, BlockSpec, LayerCall, ModelSpec
+    rms = lambda name: PartSpec("rms", {"width": D, "eps": 1e-5}, {"weight": name})
+    ln = lambda name: PartSpec("toy_layernorm", {"width": D, "eps": 1e-3}, {"weight": f"{name}.w", "bias": f"{name}.b"})
+    names = lambda p: {k: f"{p}.{k}" for k in ("q_proj", "k_proj", "v_proj", "o_proj")}
+    attn0 = PartSpec("attention", dict(hidden_size=D, n_heads=HEADS, n_kv_heads=KV, head_dim=HD,
+                                       position=PartSpec("toy_scale", {"head_dim": HD})),
+                     dict(names("b0.attn"), **{"position.freq": "b0.attn.freq"}))
+    attn1 = PartSpec("attention", dict(hidden_size=D, n_heads=HEADS, n_kv_heads=KV, head_dim=HD, visibility="window", span=6,
+                                       position=PartSpec("rotary", {"head_dim": HD, "theta": 100.0})), names("b1.attn"))
+    top2 = PartSpec("toy_top2_softmax", {"hidden_size": D, "intermediate_size": FF, "n_experts": E},
+                    {"router": "b0.ffn.router", "gate_up": "b0.ffn.gate_up", "down": "b0.ffn.down"})
+    dense = PartSpec("dense_glu", {"hidden_size": D, "intermediate_size": 40},
+                     {k: f"b1.ffn.{k}" for k in ("gate_proj", "up_proj", "down_proj")})
+    blocks = [BlockSpec("prenorm", ln("b0.n1"), attn0, ln("b0.n2"), top2),
+              BlockSpec("prenorm", rms("b1.n1"), attn1, rms("b1.n2"), dense)]
+    return ModelSpec("ToyParts", V, D, blocks, [LayerCall(0, 0), LayerCall(1, 1)], rms("final"), "embed", "head")
+
+
+def tensors(seed=0):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=g) * 0.3
+    t = {"embed": r(V, D), "head": r(V, D), "final": 1 + r(D) * 0.1, "b0.attn.freq": r(HD).abs() + 0.1}
+    for n in ("b0.n1", "b0.n2"):
+        t[f"{n}.w"], t[f"{n}.b"] = 1 + r(D) * 0.1, r(D) * 0.2
+    t["b1.n1"], t["b1.n2"] = 1 + r(D) * 0.1, 1 + r(D) * 0.1
+    for b in (0, 1):
+        t[f"b{b}.attn.q_proj"], t[f"b{b}.attn.o_proj"] = r(HEADS * HD, D), r(D, HEADS * HD)
+        t[f"b{b}.attn.k_proj"], t[f"b{b}.attn.v_proj"] = r(KV * HD, D), r(KV * HD, D)
+    t["b0.ffn.router"], t["b0.ffn.gate_up"], t["b0.ffn.down"] = r(E, D) * 3, r(E, 2 * FF, D), r(E, D, FF)
+    t["b1.ffn.gate_proj"], t["b1.ffn.up_proj"], t["b1.ffn.down_proj"] = r(40, D), r(40, D), r(D, 40)
+    return t
+
+
+def plain_toy(t, tokens):
+    """The same model, whole sequence, in float64 torch."""
+    import plain_llama4 as plain
+    W = {k: v.double() for k, v in t.items()}
+    T = len(tokens)
+    pos = torch.arange(T)
+    h = W["embed"][torch.tensor(tokens)]
+    ln = lambda x, n: F.layer_norm(x, (D,), W[f"{n}.w"], W[f"{n}.b"], 1e-3)
+    # block 0: LayerNorm, attention with the scaling encoding (full causal), LayerNorm, two experts a token
+    n = ln(h, "b0.n1")
+    s = (1 + 0.5 * torch.cos(pos.double()[:, None] * W["b0.attn.freq"][None, :]))[:, None, :]
+    q = (n @ W["b0.attn.q_proj"].T).view(T, HEADS, HD) * s
+    k = (n @ W["b0.attn.k_proj"].T).view(T, KV, HD) * s
+    v = (n @ W["b0.attn.v_proj"].T).view(T, KV, HD)
+    h = h + plain.attention(q, k, v, plain.visible_mask(pos, "full", 0)).reshape(T, HEADS * HD) @ W["b0.attn.o_proj"].T
+    n = ln(h, "b0.n2")
+    top = torch.topk(n @ W["b0.ffn.router"].T, 2, dim=-1)
+    wt = torch.softmax(top.values, dim=-1)
+    y = torch.zeros_like(h)
+    for i in range(T):
+        for c in range(2):
+            e = int(top.indices[i, c])
+            gu = W["b0.ffn.gate_up"][e] @ n[i]
+            y[i] += wt[i, c] * (W["b0.ffn.down"][e] @ (F.silu(gu[:FF]) * gu[FF:]))
+    h = h + y
+    # block 1: the built-in parts
+    n = plain.rms_norm(h, W["b1.n1"], 1e-5)
+    inv = plain.rope_inv_freq(HD, 100.0, None)
+    q = plain.apply_rope((n @ W["b1.attn.q_proj"].T).view(T, HEADS, HD), pos, inv)
+    k = plain.apply_rope((n @ W["b1.attn.k_proj"].T).view(T, KV, HD), pos, inv)
+    v = (n @ W["b1.attn.v_proj"].T).view(T, KV, HD)
+    h = h + plain.attention(q, k, v, plain.visible_mask(pos, "window", 6)).reshape(T, HEADS * HD) @ W["b1.attn.o_proj"].T
+    h = h + plain.swiglu_mlp(plain.rms_norm(h, W["b1.n2"], 1e-5), W["b1.ffn.gate_proj"], W["b1.ffn.up_proj"], W["b1.ffn.down_proj"])
+    return (plain.rms_norm(h, W["final"], 1e-5) @ W["head"].T).float().numpy()
+
+
+def test_other_norms_position_encodings_and_routed_feed_forwards_are_built_and_stepped():
+    from spite_amd import Engine
+    from spite_amd.parts import registered
+    define_parts()
+    assert "toy_layernorm" in registered("norm") and "toy_scale" in registered("position") \
+        and "toy_top2_softmax" in registered("ffn")
+    t = tensors()
+    eng = Engine(spec=spec(), tensors=t, dtype="float32", page_size=4, cache_tokens=96, max_requests=3)
+    assert not eng.use_graphs                     # the toy parts do not claim to be safe to capture
+    assert eng.cache.n_groups() == 2              # a full group and a window group
+    reqs = {"x": H.random_tokens(V, 23, 1), "y": H.random_tokens(V, 9, 2), "z": H.random_tokens(V, 15, 3)}
+    ref = {(rid, i): row for rid, toks in reqs.items() for i, row in enumerate(plain_toy(t, toks))}
+    for steps in (H.schedule_whole(reqs), H.schedule_tail_one_by_one(reqs, tail=8),
+                  H.schedule_portions(reqs, sizes=(3, 2, 7, 2)), H.schedule_mixed(reqs, seed=4, max_live=3)):
+        got = H.collect(steps, H.run_trace_inprocess(eng, steps), V)
+        d, where = H.max_diff(got, ref)
+        assert d < 1e-4, (d, where)
+
+
+def test_the_same_toy_parts_in_bfloat16():
+    """bfloat16 activations and weights through the same parts: the grouped MFMA products take the
+    toy feed-forward's row list (two slots a token, weights on the output)."""
+    from spite_amd import Engine
+    define_parts()
+    t16 = {k: v.to(torch.bfloat16) for k, v in tensors().items()}        # a bfloat16 checkpoint
+    t = {k: v.float() for k, v in t16.items()}
+    eng = Engine(spec=spec(), tensors=t16, dtype="bfloat16", page_size=4, cache_tokens=96, max_requests=3)
+    reqs = {"x": H.random_tokens(V, 23, 1)}
+    ref = plain_toy(t, reqs["x"])
+    got = H.collect(H.schedule_whole(reqs), H.run_trace_inprocess(eng, H.schedule_whole(reqs)), V)
+    err = max(abs(got[("x", i)] - ref[i]).max() for i in range(23))
+    # an expert chosen differently at a near tie of the router would show as an error of the
+    # logits' own size; rounding to bfloat16 along two layers stays a few percent of it
+    assert err < 0.06 * abs(ref).max(), (err, abs(ref).max())
