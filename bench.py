@@ -52,12 +52,17 @@ def layer_bytes(cfg, item=2):
 
 
 def decode_bytes(cfg, L, batch, context, experts_touched, item=2):
-    """Bytes one decode step has to read: every weight it uses once and the live cache."""
+    """Bytes one decode step has to read: every weight it uses once and the cache that the live
+    requests' queries can see (every fourth layer the whole context, the others the current
+    chunk)."""
     d, V = cfg["hidden_size"], cfg["vocab_size"]
     attn, expert, small = layer_bytes(cfg, item)
     kv_token = 2 * cfg["num_key_value_heads"] * cfg["head_dim"] * item
-    per_layer = attn + small + expert * (1 + experts_touched) + batch * context * kv_token
-    return L * per_layer + V * d * item + batch * d * item + d * 4
+    chunk = cfg["attention_chunk_size"]
+    n_full = sum(1 for layer in range(L) if (layer + 1) % 4 == 0)
+    seen = n_full * context + (L - n_full) * (context % chunk + 1 if context >= chunk else context)
+    return L * (attn + small + expert * (1 + experts_touched)) + batch * seen * kv_token \
+        + V * d * item + batch * d * item + d * 4
 
 
 def prefill_flops(cfg, L, T):
@@ -191,7 +196,7 @@ def main() -> int:
         log(f"decode batch {b}: {d_b / n * 1e3:.2f} ms/step")
 
     out = {
-        "metric": "decode tok/s at batch 8, context 4096 (Llama 4 Scout shape, random weights)",
+        "metric": f"decode tok/s at batch {args.batch}, context {args.context} (Llama 4 Scout shape, random weights)",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic: random weights N(0,0.02), uniform-random token ids, "
