@@ -401,8 +401,17 @@ extern "C" int spite_router_top1(const float* x, const float* wr, int* expert, f
 // expert[] and weight[]: the largest logit, the lowest index among equals, weight =
 // 1/(1+exp(-logit)).
 __device__ __forceinline__ int top1_of(const float* __restrict__ l, int E, float* best_out) {
-    float best = l[0]; int best_e = 0;
-    for (int e = 1; e < E; ++e) { const float v = l[e]; if (v > best) { best = v; best_e = e; } }
+    float best = -INFINITY; int best_e = 0;
+    if ((E & 3) == 0 && (((uintptr_t)l) & 15) == 0) {           // four logits a load
+        for (int e = 0; e < E; e += 4) {
+            const f32x4 v = *(const f32x4*)(l + e);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) if (v[i] > best || (e + i == 0)) { best = v[i]; best_e = e + i; }
+        }
+    } else {
+        best = l[0];
+        for (int e = 1; e < E; ++e) { const float v = l[e]; if (v > best) { best = v; best_e = e; } }
+    }
     if (best_out) *best_out = best;
     return best_e;
 }
