@@ -16,6 +16,11 @@
 // applied per element from the column's position and the key's; blocks that every column of
 // a wave sees whole skip the tests, blocks that none sees are skipped.
 //
+// KS = 2 (short prompts, where a tile's walk over its keys is the longest path and there are
+// too few tiles to fill the chip): the tile has half the columns, waves 0-3 take them on the
+// even blocks of 64 keys and waves 4-7 the same columns on the odd blocks; two blocks are staged
+// per step, and at the end the two halves' (maximum, sum, output) meet in LDS.
+//
 // Order of keys.  The score product leaves lane (n, qd) with rows qd*4 .. qd*4+3 of each
 // 16-row tile; the second product wants 8 consecutive k indices per lane.  The rows qd*4+i of
 // the two tiles of a 32-key half are therefore the keys qd*8 + i and qd*8 + 4 + i: a lane's
@@ -27,10 +32,10 @@
 // MFMA operand.
 #include "common.h"
 
-#define PF_COLS 256        // columns (query, head) per workgroup
+#define PF_COLS 256        // columns (query, head) per workgroup (divided by KS)
 #define PF_KEYS 64         // keys per block
 
-template <int HD>
+template <int HD, int KS>
 __global__ __launch_bounds__(512)
 void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages,
                          const bf16* __restrict__ v_pages, bf16* __restrict__ out,
@@ -38,13 +43,14 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
                          const int* __restrict__ block_table, int max_blocks, int tile_q,
                          int H, int G, int ps, int vis, int span, float scale_log2e) {
     constexpr int NC = HD / 32, ND = HD / 16;
-    constexpr int KCH = PF_KEYS * HD / 8 / 512;      // 16-byte chunks of the K block per thread
-    constexpr int VCH = HD * PF_KEYS / 8 / 512;      // and of the V^T block
+    constexpr int KCH = KS * PF_KEYS * HD / 8 / 512; // 16-byte chunks of the step's K blocks per thread
+    constexpr int VCH = KCH;                         // and of its V^T blocks
     constexpr int KHALF = 2 * NC * 64;               // chunks of one 32-key half of a K block
-    constexpr int VHALF = ND * 64;                   // and of a V^T block
+    constexpr int VHALF = ND * 64;                   // and of a V^T block (the same number)
+    constexpr int STEP = KS * PF_KEYS * HD;          // elements of the K (or V^T) blocks of one step
     extern __shared__ __attribute__((aligned(16))) bf16 sm[];
-    bf16* Ks = sm;                                   // [2][half][tile tt][chunk cc][512]
-    bf16* Vs = sm + 2 * PF_KEYS * HD;                // [2][half][tile d][512]
+    bf16* Ks = sm;                                   // [2 buffers][KS blocks][half][tile tt][chunk cc][512]
+    bf16* Vs = sm + 2 * STEP;                        // [2 buffers][KS blocks][half][tile d][512]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, qd = lane >> 4;
@@ -63,6 +69,8 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
     const int* bt = block_table + (size_t)seq * max_blocks;
     const int p_first = positions[t0], p_last = positions[t_end - 1];
     const int b_first = sp_first_visible(p_first, vis, span) / PF_KEYS, b_last = p_last / PF_KEYS;
+    const int wcol = KS == 2 ? (wave & 3) : wave;    // which 32 columns; with KS = 2 waves w and w+4 share them
+    const int khalf = KS == 2 ? (wave >> 2) : 0;     // and take the even (0) or the odd (1) blocks
 
     // this lane's two columns
     int pq[2], lo[2], tok[2], head[2];
@@ -71,7 +79,7 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
     int pq_min = 0x7fffffff, pq_max = -1, lo_min = 0x7fffffff, lo_max = 0;
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
-        const int col = wave * 32 + c * 16 + n;
+        const int col = wcol * 32 + c * 16 + n;
         const int tq = col / QH;
         tok[c] = t0 + tq;
         head[c] = g * QH + col % QH;
@@ -106,41 +114,45 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
 
     // ---- staging: thread's chunks of the block, pages -> registers -> LDS
     bf16x8 kreg[KCH], vreg[VCH];
-    auto stage_load = [&](int kb) {
-        const int key0 = kb * PF_KEYS;
-        const int pg0 = page_of(key0), pg1 = page_of(key0 + 32);
-        const int blk0 = (key0 % ps) >> 5, blk1 = ((key0 + 32) % ps) >> 5;     // the 32-key blocks inside their pages
-        // pages that are absent are read as page 0: their keys are masked, or poisoned below
-        const size_t slab0 = ((size_t)(pg0 < 0 ? 0 : pg0) * G + g) * (size_t)ps * HD;
-        const size_t slab1 = ((size_t)(pg1 < 0 ? 0 : pg1) * G + g) * (size_t)ps * HD;
+    // step u stages the blocks u*KS .. u*KS + KS-1; every 32-key half comes from its own page
+    auto stage_load = [&](int u) {
+        size_t base[2 * KS];
+#pragma unroll
+        for (int h = 0; h < 2 * KS; ++h) {
+            const int key = (u * KS) * PF_KEYS + h * 32;
+            const int pg = page_of(key);
+            // pages that are absent are read as page 0: their keys are masked, or poisoned below
+            base[h] = ((size_t)(pg < 0 ? 0 : pg) * G + g) * (size_t)ps * HD + (size_t)((key % ps) >> 5) * (KHALF * 8);
+        }
 #pragma unroll
         for (int i = 0; i < KCH; ++i) {
             const int c = tid + 512 * i;
-            const size_t at = c < KHALF ? slab0 + ((size_t)blk0 * KHALF + c) * 8 : slab1 + ((size_t)blk1 * KHALF + (c - KHALF)) * 8;
-            kreg[i] = *(const bf16x8*)(k_pages + at);
-        }
+            const int h = c / KHALF;                 // which half of which block: a constant where KHALF >= 512
+            size_t at = base[0];
 #pragma unroll
-        for (int i = 0; i < VCH; ++i) {
-            const int c = tid + 512 * i;
-            const size_t at = c < VHALF ? slab0 + ((size_t)blk0 * VHALF + c) * 8 : slab1 + ((size_t)blk1 * VHALF + (c - VHALF)) * 8;
-            vreg[i] = *(const bf16x8*)(v_pages + at);
+            for (int hh = 1; hh < 2 * KS; ++hh) at = h == hh ? base[hh] : at;
+            at += (size_t)(c - h * KHALF) * 8;
+            kreg[i] = *(const bf16x8*)(k_pages + at);
+            vreg[i] = *(const bf16x8*)(v_pages + at);      // V^T tiles of a half lie where its K tiles do
         }
     };
     auto stage_store = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < KCH; ++i) *(bf16x8*)(Ks + buf * PF_KEYS * HD + (tid + 512 * i) * 8) = kreg[i];
-#pragma unroll
-        for (int i = 0; i < VCH; ++i) *(bf16x8*)(Vs + buf * HD * PF_KEYS + (tid + 512 * i) * 8) = vreg[i];
+        for (int i = 0; i < KCH; ++i) {
+            *(bf16x8*)(Ks + buf * STEP + (tid + 512 * i) * 8) = kreg[i];
+            *(bf16x8*)(Vs + buf * STEP + (tid + 512 * i) * 8) = vreg[i];
+        }
     };
 
     // ---- one block of 64 keys out of LDS
     auto compute = [&](int kb, int buf) {
+        if (kb < b_first || kb > b_last) return;
         const int key0 = kb * PF_KEYS;
         if (key0 > pq_max || key0 + PF_KEYS - 1 < lo_min) return;     // nothing here for this wave
         const bool whole = key0 >= lo_max && key0 + PF_KEYS - 1 <= pq_min;
         const bool absent0 = page_of(key0) < 0, absent1 = page_of(key0 + 32) < 0;
-        const bf16* kb_ = Ks + buf * PF_KEYS * HD + lane * 8;
-        const bf16* vb_ = Vs + buf * HD * PF_KEYS + lane * 8;
+        const bf16* kb_ = Ks + buf * STEP + khalf * PF_KEYS * HD + lane * 8;
+        const bf16* vb_ = Vs + buf * STEP + khalf * PF_KEYS * HD + lane * 8;
         f32x4 s[2][4];
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) {
@@ -159,14 +171,9 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
         float alpha[2];
 #pragma unroll
         for (int c = 0; c < 2; ++c) {
-            float mx = -INFINITY;
-            // s[c][tt][i] is the key key0 + (tt/2)*32 + qd*8 + (tt%2)*4 + i
-            if (whole && !absent0 && !absent1) {
-#pragma unroll
-                for (int tt = 0; tt < 4; ++tt)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) { s[c][tt][i] *= scale_log2e; mx = fmaxf(mx, s[c][tt][i]); }
-            } else {
+            // s[c][tt][i] is the key key0 + (tt/2)*32 + qd*8 + (tt%2)*4 + i; keys that the column
+            // may not read become -inf, keys of a page that was given back NaN
+            if (!(whole && !absent0 && !absent1)) {
 #pragma unroll
                 for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
@@ -174,23 +181,27 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
                         const int j = key0 + (tt >> 1) * 32 + qd * 8 + (tt & 1) * 4 + i;
                         const bool ok = j >= lo[c] && j <= pq[c];
                         const bool absent = (tt >> 1) ? absent1 : absent0;
-                        const float v = ok ? (absent ? NAN : s[c][tt][i] * scale_log2e) : -INFINITY;
-                        s[c][tt][i] = v;
-                        mx = fmaxf(mx, v);
+                        s[c][tt][i] = ok ? (absent ? NAN : s[c][tt][i]) : -INFINITY;
                     }
             }
+            // the maximum of the raw scores; the scale (positive) goes into the exponent's fma
+            float mx = -INFINITY;
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s[c][tt][i]);
             mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            const float m_new = fmaxf(m_run[c], mx);
+            const float m_new = fmaxf(m_run[c], mx * scale_log2e);
             // a column with nothing visible so far keeps m = -inf: its weights are zero, not NaN
             const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-            alpha[c] = exp2f(m_run[c] - m_safe);
+            alpha[c] = __builtin_amdgcn_exp2f(m_run[c] - m_safe);
             float sum = 0.f;
 #pragma unroll
             for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const float e = exp2f(s[c][tt][i] - m_safe);
+                    const float e = __builtin_amdgcn_exp2f(fmaf(s[c][tt][i], scale_log2e, -m_safe));
                     sum += e;
                     pf[c][tt >> 1][(tt & 1) * 4 + i] = (bf16)e;
                 }
@@ -199,10 +210,15 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
             l_run[c] = l_run[c] * alpha[c] + sum;
             m_run[c] = m_new;
         }
+        // the running maxima move in the first blocks and seldom after: the output is rescaled
+        // only when some column of the wave needs it (alpha is exactly 1 otherwise)
+        const bool rescale = __any(alpha[0] != 1.0f || alpha[1] != 1.0f);
 #pragma unroll
         for (int d = 0; d < ND; ++d) {
+            if (rescale) {
 #pragma unroll
-            for (int c = 0; c < 2; ++c) o[c][d] = o[c][d] * alpha[c];
+                for (int c = 0; c < 2; ++c) o[c][d] = o[c][d] * alpha[c];
+            }
 #pragma unroll
             for (int hh = 0; hh < 2; ++hh) {
                 const bf16x8 vf = *(const bf16x8*)(vb_ + (hh * ND + d) * 512);
@@ -213,15 +229,50 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
         }
     };
 
-    stage_load(b_first);
+    const int u_first = b_first / KS, u_last = b_last / KS;
+    stage_load(u_first);
     stage_store(0);
     __syncthreads();
-    for (int kb = b_first; kb <= b_last; ++kb) {
-        const int buf = (kb - b_first) & 1;
-        if (kb < b_last) stage_load(kb + 1);
-        compute(kb, buf);
-        if (kb < b_last) stage_store(buf ^ 1);
+    for (int u = u_first; u <= u_last; ++u) {
+        const int buf = (u - u_first) & 1;
+        if (u < u_last) stage_load(u + 1);
+        compute(u * KS + khalf, buf);
+        if (u < u_last) stage_store(buf ^ 1);
         __syncthreads();
+    }
+
+    if (KS == 2) {
+        // the odd blocks' results join the even blocks': per lane 2 maxima, 2 sums and the output,
+        // laid out [item][wave of the pair][lane] so that a wave's accesses run through the banks
+        float* xs = (float*)sm;
+        constexpr int ITEMS = 4 + 2 * ND * 4;
+        float* mine = xs + ((size_t)wcol * 64 + lane);
+        auto at = [&](int item) -> float& { return mine[(size_t)item * 256]; };
+        if (khalf == 1) {
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                at(c) = m_run[c]; at(2 + c) = l_run[c];
+#pragma unroll
+                for (int d = 0; d < ND; ++d)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) at(4 + (c * ND + d) * 4 + i) = o[c][d][i];
+            }
+        }
+        __syncthreads();
+        if (khalf == 1) return;
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const float mb = at(c), lb = at(2 + c);
+            const float M = fmaxf(m_run[c], mb);
+            const float fa = (m_run[c] == -INFINITY) ? 0.f : exp2f(m_run[c] - M);
+            const float fb = (mb == -INFINITY) ? 0.f : exp2f(mb - M);
+            l_run[c] = fa * l_run[c] + fb * lb;
+#pragma unroll
+            for (int d = 0; d < ND; ++d)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) o[c][d][i] = fa * o[c][d][i] + fb * at(4 + (c * ND + d) * 4 + i);
+        }
+        (void)ITEMS;
     }
 
     // o[c][d][i] of lane (n, qd): column c*16 + n of the wave, element d*16 + qd*4 + i
@@ -240,48 +291,56 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
     }
 }
 
+template <int HD, int KS>
+static int launch_prefill(const void* q, const void* k_pages, const void* v_pages, void* out, const int* positions,
+                          const int* cu_seqlens, int n_seqs, const int* block_table, int max_blocks, int tile_q,
+                          long n_tiles, int H, int G, int page_size, int vis, int span, float sl, hipStream_t st) {
+    const size_t sh = (size_t)2 * 2 * KS * PF_KEYS * HD * sizeof(bf16);
+    static bool allowed = false;          // one flag per instantiation: more LDS than the default limit
+    if (!allowed) {
+        hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_kernel<HD, KS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sh);
+        SP_REQUIRE(e == hipSuccess, "attn_prefill: %zu bytes of LDS refused: %s", sh, hipGetErrorString(e));
+        allowed = true;
+    }
+    attn_prefill_kernel<HD, KS><<<dim3((unsigned)n_tiles, G), 512, sh, st>>>((const bf16*)q, (const bf16*)k_pages,
+        (const bf16*)v_pages, (bf16*)out, positions, cu_seqlens, n_seqs, block_table, max_blocks, tile_q, H, G, page_size,
+        vis, span, sl);
+    SP_LAUNCH_CHECK("attn_prefill");
+    return 0;
+}
+
 // `counts` (host memory): the number of query tokens of each of the step's `n_seqs` requests,
-// in the order of `cu_seqlens` (device), whose differences they are.
+// in the order of `cu_seqlens` (device), whose differences they are.  `key_split`: 0 lets the
+// library choose, 1 or 2 force KS.
 extern "C" int spite_attn_prefill(const void* q, const void* k_pages, const void* v_pages, void* out,
                                   const int* positions, const int* cu_seqlens, const int* counts, int n_seqs,
                                   const int* block_table, int max_blocks, int H, int G, int hd, int page_size,
-                                  int vis, int span, float scale, hipStream_t st) {
+                                  int vis, int span, float scale, int key_split, hipStream_t st) {
     SP_REQUIRE(n_seqs >= 0 && H > 0 && G > 0 && H % G == 0, "attn_prefill: %d query heads over %d kv heads", H, G);
-    SP_REQUIRE(H / G <= PF_COLS, "attn_prefill: %d query heads per kv head, at most %d", H / G, PF_COLS);
+    SP_REQUIRE(H / G <= PF_COLS / 2, "attn_prefill: %d query heads per kv head, at most %d", H / G, PF_COLS / 2);
     SP_REQUIRE(hd == 64 || hd == 128, "attn_prefill: head size %d (this kernel has 64 and 128)", hd);
     SP_REQUIRE(page_size > 0 && page_size % 32 == 0, "attn_prefill: page size %d must be a multiple of 32", page_size);
     SP_REQUIRE(max_blocks > 0, "attn_prefill: bad table width");
     SP_REQUIRE(vis == SP_VIS_FULL || span > 0, "attn_prefill: chunk or window of %d", span);
     SP_REQUIRE(G <= 65535, "attn_prefill: too many kv heads for one launch");
-    const int tile_q = PF_COLS / (H / G);
-    long n_tiles = 0;
-    for (int s = 0; s < n_seqs; ++s) {
-        SP_REQUIRE(counts[s] >= 0, "attn_prefill: request %d with %d tokens", s, counts[s]);
-        n_tiles += (counts[s] + tile_q - 1) / tile_q;
+    SP_REQUIRE(key_split >= 0 && key_split <= 2, "attn_prefill: key split %d", key_split);
+    long tiles[3] = {0, 0, 0};
+    for (int ks = 1; ks <= 2; ++ks) {
+        const int tile_q = PF_COLS / ks / (H / G);
+        for (int s = 0; s < n_seqs; ++s) {
+            SP_REQUIRE(counts[s] >= 0, "attn_prefill: request %d with %d tokens", s, counts[s]);
+            tiles[ks] += (counts[s] + tile_q - 1) / tile_q;
+        }
     }
-    if (n_tiles == 0) return 0;
-    SP_REQUIRE(n_tiles <= 0x7fffffffL, "attn_prefill: too many tiles");
+    if (tiles[1] == 0) return 0;
+    // few tiles: the longest tile's walk decides the time, so halve it
+    if (key_split == 0) key_split = tiles[1] * G < 512 ? 2 : 1;
+    SP_REQUIRE(tiles[key_split] <= 0x7fffffffL, "attn_prefill: too many tiles");
     const float sl = scale * 1.4426950408889634f;
-    dim3 grid((unsigned)n_tiles, G);
-    const size_t sh = (size_t)2 * 2 * PF_KEYS * hd * sizeof(bf16);
-    static bool allowed[2] = {false, false};     // the kernels ask for more LDS than the default limit
-    if (hd == 128) {
-        if (!allowed[0]) {
-            hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sh);
-            SP_REQUIRE(e == hipSuccess, "attn_prefill: %zu bytes of LDS refused: %s", sh, hipGetErrorString(e));
-            allowed[0] = true;
-        }
-        attn_prefill_kernel<128><<<grid, 512, sh, st>>>((const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages,
-            (bf16*)out, positions, cu_seqlens, n_seqs, block_table, max_blocks, tile_q, H, G, page_size, vis, span, sl);
-    } else {
-        if (!allowed[1]) {
-            hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sh);
-            SP_REQUIRE(e == hipSuccess, "attn_prefill: %zu bytes of LDS refused: %s", sh, hipGetErrorString(e));
-            allowed[1] = true;
-        }
-        attn_prefill_kernel<64><<<grid, 512, sh, st>>>((const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages,
-            (bf16*)out, positions, cu_seqlens, n_seqs, block_table, max_blocks, tile_q, H, G, page_size, vis, span, sl);
-    }
-    SP_LAUNCH_CHECK("attn_prefill");
-    return 0;
+    const int tile_q = PF_COLS / key_split / (H / G);
+#define SP_PF(HDV, KSV) launch_prefill<HDV, KSV>(q, k_pages, v_pages, out, positions, cu_seqlens, n_seqs, block_table, \
+        max_blocks, tile_q, tiles[KSV], H, G, page_size, vis, span, sl, st)
+    if (hd == 128) return key_split == 2 ? SP_PF(128, 2) : SP_PF(128, 1);
+    return key_split == 2 ? SP_PF(64, 2) : SP_PF(64, 1);
+#undef SP_PF
 }

@@ -46,7 +46,7 @@ def lib():
             "spite_attn_decode": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, P],
             "spite_gemm_mfma": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, P],
             "spite_gemm_tiled": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, P],
-            "spite_attn_prefill": [P, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, F, P],
+            "spite_attn_prefill": [P, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, F, I, P],
             "spite_argmax_rows": [P, I, I, I, P, P, P, P],
         }
         for name, args in sigs.items():
@@ -388,7 +388,7 @@ def gemm_tiled(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_sca
 
 
 def attn_prefill(q, k_pages, v_pages, out, positions, cu_seqlens, counts, block_table,
-                 H, G, hd, page_size, vis, span, scale):
+                 H, G, hd, page_size, vis, span, scale, key_split=0):
     """Prefill attention on MFMA (bf16; head sizes 64 and 128; pages of a multiple of 32 keys, in
     operand order).
     ``counts``: the number of query tokens of every request of the step, on the host, in the
@@ -410,7 +410,7 @@ def attn_prefill(q, k_pages, v_pages, out, positions, cu_seqlens, counts, block_
         _ptr(q, "q", dt), _ptr(k_pages, "k_pages", dt), _ptr(v_pages, "v_pages", dt), _ptr(out, "out", dt),
         _ptr(positions, "positions", torch.int32), _ptr(cu_seqlens, "cu_seqlens", torch.int32),
         counts.ctypes.data, n_seqs, _ptr(block_table, "block_table", torch.int32), block_table.shape[1],
-        H, G, hd, page_size, VIS[vis], int(span or 0), float(scale), _stream()), "attn_prefill")
+        H, G, hd, page_size, VIS[vis], int(span or 0), float(scale), int(key_split), _stream()), "attn_prefill")
 
 
 def argmax_rows(logits, out, scratch_v, scratch_i, n_rows=None):

@@ -389,8 +389,9 @@ PORTION_CASES = [
 ]
 
 
+@pytest.mark.parametrize("key_split", [1, 2])
 @pytest.mark.parametrize("case", PORTION_CASES, ids=lambda c: f"H{c[0]}G{c[1]}hd{c[2]}ps{c[3]}{c[6]}")
-def test_attn_prefill(case):
+def test_attn_prefill(case, key_split):
     H, G, hd, ps, lens, portions, vis, span = case
     dtype = torch.bfloat16
     kv = PagedKV(lens, G, hd, ps, dtype, seed=3)
@@ -410,7 +411,7 @@ def test_attn_prefill(case):
     out = torch.zeros(T, H * hd, dtype=dtype, device=DEV)
     ops().attn_prefill(qs.reshape(T, H * hd).to(DEV), *ops().kv_operand_order(kv.kp.to(DEV), kv.vp.to(DEV)), out, positions,
                        torch.tensor(cu, dtype=torch.int32, device=DEV), [count for _, _, count in portions], bt,
-                       H, G, hd, ps, vis, span, 1.0 / math.sqrt(hd))
+                       H, G, hd, ps, vis, span, 1.0 / math.sqrt(hd), key_split=key_split)
     got = out.double().cpu().view(T, H, hd)
     assert torch.isfinite(got).all()
     assert (got - ref).abs().max() < 1.5e-2 * max(1.0, float(ref.abs().max()))
