@@ -264,6 +264,110 @@ void rope_kvwrite_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
     }
 }
 
+// The same for bfloat16 rows whose head size gives every head a power-of-two group of lanes with
+// four pairs each (hd = 32, 64, 128, 256, 512): a lane reads and writes eight bytes at a time
+// instead of two, and a wave handles 64 / (hd/8) heads at once.  Every value is computed by the
+// same operations in the same order as in the kernel above; only the sum of squares of the
+// qk-norm meets in a different order.
+__global__ __launch_bounds__(256)
+void rope_kvwrite_vec_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ q_out,
+                             bf16* __restrict__ k_pages, bf16* __restrict__ v_pages,
+                             const int* __restrict__ positions, const int* __restrict__ slot_map,
+                             const float* __restrict__ inv_freq, int H, int G, int hd, int ps,
+                             int use_rope, int adjacent, int use_norm, float norm_eps,
+                             int use_temp, int floor_scale, float attn_scale, int n_heads, int hpw, int kv_tiled) {
+    const int t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int half = hd >> 1;
+    const int lph = half >> 2;                   // lanes a head: four pairs each
+    const int sub = lane / lph, l = lane % lph;  // which head of the wave's group, which four pairs
+    const int hpi = 64 / lph;                    // heads a wave takes at once
+    const int row_w = (H + 2 * G) * hd;
+    const int pos = positions[t];
+    const int slot = slot_map ? slot_map[t] : -1;
+    float sn[4], cs[4];
+    if (use_rope) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) sincosf((float)pos * inv_freq[4 * l + u], &sn[u], &cs[u]);
+    }
+    float temp = 1.f;
+    if (use_temp) temp = logf((float)((pos + 1) / floor_scale) + 1.0f) * attn_scale + 1.0f;
+
+    for (int it = 0; it < hpw; ++it) {
+        const int hh = (blockIdx.y * 4 * hpw + it * 4 + wave) * hpi + sub;
+        const bool have = hh < n_heads;          // lanes past the last head idle, but join the shuffles
+        const bf16* src = qkv + (size_t)t * row_w + (size_t)(have ? hh : 0) * hd;
+        const bool is_q = hh < H;
+        const bool is_v = hh >= H + G;
+        const int g = is_v ? hh - H - G : hh - H;
+        const size_t page = slot >= 0 ? slot / ps : 0;
+        const int off = slot >= 0 ? slot % ps : 0;
+        // the four pairs' elements: half-split (4l+u, half+4l+u) or adjacent (8l+2u, 8l+2u+1)
+        bf16x4 lo4 = *(const bf16x4*)(src + (adjacent ? 8 * l : 4 * l));
+        bf16x4 hi4 = *(const bf16x4*)(src + (adjacent ? 8 * l + 4 : half + 4 * l));
+        if (have && is_v) {
+            if (slot >= 0) {
+                bf16* slab = v_pages + (page * G + g) * (size_t)hd * ps;
+                const int c0 = adjacent ? 8 * l : 4 * l, c1 = adjacent ? 8 * l + 4 : half + 4 * l;
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    slab[sp_v_index(c0 + u, off, hd, ps, kv_tiled)] = lo4[u];
+                    slab[sp_v_index(c1 + u, off, hd, ps, kv_tiled)] = hi4[u];
+                }
+            }
+        }
+        float x0[4], x1[4];
+        float ss = 0.f;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            float a, b;
+            if (adjacent) {              // pairs (8l+2u, 8l+2u+1): two from lo4, two from hi4
+                a = (float)(u < 2 ? lo4[2 * u] : hi4[2 * u - 4]);
+                b = (float)(u < 2 ? lo4[2 * u + 1] : hi4[2 * u - 3]);
+            } else {
+                a = (float)lo4[u]; b = (float)hi4[u];
+            }
+            if (use_rope) {
+                const int su = adjacent ? u : u;
+                // adjacent pairing: pair index 4l+u as well
+                const float ra = a * cs[su] - b * sn[su];
+                const float rb = a * sn[su] + b * cs[su];
+                a = ra; b = rb;
+            }
+            x0[u] = a; x1[u] = b;
+            ss += a * a + b * b;
+        }
+        float scale = 1.f;
+        if (use_norm) {
+            for (int o = 1; o < lph; o <<= 1) ss += __shfl_xor(ss, o, 64);
+            scale = 1.0f / sqrtf(ss / (float)hd + norm_eps);
+        }
+        if (is_q) scale *= temp;
+        if (!have || is_v || (!is_q && slot < 0)) continue;
+        bf16x4 o_lo, o_hi;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const bf16 ya = (bf16)(x0[u] * scale), yb = (bf16)(x1[u] * scale);
+            if (adjacent) {
+                if (u < 2) { o_lo[2 * u] = ya; o_lo[2 * u + 1] = yb; } else { o_hi[2 * u - 4] = ya; o_hi[2 * u - 3] = yb; }
+            } else {
+                o_lo[u] = ya; o_hi[u] = yb;
+            }
+        }
+        const int c0 = adjacent ? 8 * l : 4 * l, c1 = adjacent ? 8 * l + 4 : half + 4 * l;
+        if (is_q) {
+            bf16* dst = q_out + ((size_t)t * H + hh) * hd;
+            *(bf16x4*)(dst + c0) = o_lo;
+            *(bf16x4*)(dst + c1) = o_hi;
+        } else {
+            bf16* slab = k_pages + (page * G + g) * (size_t)ps * hd;
+            // four elements in a row stay in a row in operand order too (they share a group of eight)
+            *(bf16x4*)(slab + sp_k_index(off, c0, hd, kv_tiled)) = o_lo;
+            *(bf16x4*)(slab + sp_k_index(off, c1, hd, kv_tiled)) = o_hi;
+        }
+    }
+}
+
 extern "C" int spite_rope_kvwrite(const void* qkv, void* q_out, void* k_pages, void* v_pages, int dtype,
                                   const int* positions, const int* slot_map, const float* inv_freq,
                                   int T, int H, int G, int hd, int page_size, int use_rope, int adjacent,
@@ -281,6 +385,18 @@ extern "C" int spite_rope_kvwrite(const void* qkv, void* q_out, void* k_pages, v
     if (T == 0) return 0;
     const int n_heads = write_kv ? H + 2 * G : H;
     const int hpw = T >= 256 ? 4 : 1;            // many tokens: fewer, longer workgroups
+    const int lph = hd / 8;                      // lanes a head in the 8-byte kernel
+    auto al8 = [](const void* p) { return ((uintptr_t)p & 7) == 0; };
+    if (dtype == SP_BF16 && hd % 8 == 0 && lph >= 1 && lph <= 64 && (lph & (lph - 1)) == 0 && al8(qkv) && al8(q_out)
+        && al8(k_pages) && (page_size % 4 == 0 || !write_kv)) {
+        const int hpi = 64 / lph;
+        dim3 grid(T, (n_heads + 4 * hpw * hpi - 1) / (4 * hpw * hpi));
+        rope_kvwrite_vec_kernel<<<grid, 256, 0, st>>>((const bf16*)qkv, (bf16*)q_out, (bf16*)k_pages, (bf16*)v_pages,
+            positions, slot_map, inv_freq, H, G, hd, page_size, use_rope, adjacent, use_norm, norm_eps, use_temp,
+            floor_scale, attn_scale, n_heads, hpw, kv_tiled);
+        SP_LAUNCH_CHECK("rope_kvwrite");
+        return 0;
+    }
     dim3 grid(T, (n_heads + 4 * hpw - 1) / (4 * hpw));
     if (dtype == SP_F32)
         rope_kvwrite_kernel<float><<<grid, 256, 0, st>>>((const float*)qkv, (float*)q_out, (float*)k_pages,
