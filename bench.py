@@ -212,6 +212,7 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK, 4)},
         "points": pts,
+        "peak_memory_gib": round(torch.cuda.max_memory_allocated() / 2**30, 1),
     }
     print(json.dumps(out))
     return 0
