@@ -61,16 +61,23 @@ def decode_bytes(cfg, L, batch, context, experts_touched, item=2):
     chunk = cfg["attention_chunk_size"]
     n_full = sum(1 for layer in range(L) if (layer + 1) % 4 == 0)
     seen = n_full * context + (L - n_full) * (context % chunk + 1 if context >= chunk else context)
-    return L * (attn + small + expert * (1 + experts_touched)) + batch * seen * kv_token \
-        + V * d * item + batch * d * item + d * 4
+    step = cfg["interleave_moe_layer_step"]
+    n_moe = sum(1 for layer in range(L) if (layer + 1) % step == 0)
+    dense = 3 * d * cfg["intermediate_size_mlp"] * item
+    return L * (attn + small) + n_moe * expert * (1 + experts_touched) + (L - n_moe) * dense \
+        + batch * seen * kv_token + V * d * item + batch * d * item + d * 4
 
 
 def prefill_flops(cfg, L, T):
     d, H, G, hd = cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
     F, V = cfg["intermediate_size"], cfg["vocab_size"]
-    proj = (H + 2 * G) * hd * d + d * H * hd + 2 * 3 * d * F + cfg["num_local_experts"] * d
+    step = cfg["interleave_moe_layer_step"]
+    n_moe = sum(1 for layer in range(L) if (layer + 1) % step == 0)
+    proj = (H + 2 * G) * hd * d + d * H * hd
+    moe = 2 * 3 * d * F + cfg["num_local_experts"] * d            # one routed expert and the shared one a token
+    dense = 3 * d * cfg["intermediate_size_mlp"]
     attn = 4 * (T * (T + 1) // 2) * H * hd
-    return L * (2 * proj * T + attn) + 2 * d * V
+    return L * (2 * proj * T + attn) + 2 * T * (n_moe * moe + (L - n_moe) * dense) + 2 * d * V
 
 
 def main() -> int:
@@ -85,6 +92,9 @@ def main() -> int:
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--tiny", action="store_true", help="a small model of the same kind, to try the script")
+    ap.add_argument("--experts", type=int, default=None, help="routed experts a layer (default: the model's 16)")
+    ap.add_argument("--moe-step", type=int, default=None,
+                    help="every how many layers the feed-forward is the experts' (default 1; 2 = dense layers between)")
     ap.add_argument("--no-graphs", action="store_true", help="run decode steps eagerly (for kernel traces)")
     ap.add_argument("--phase", default="all", choices=["all", "decode", "prefill"],
                     help="time only one phase (for kernel traces); the other's figures are null")
@@ -102,6 +112,10 @@ def main() -> int:
     layers_full = base["num_hidden_layers"]
     L = args.layers or layers_full
     cfg = dict(base, num_hidden_layers=L, no_rope_layers=None)
+    if args.experts:
+        cfg["num_local_experts"] = args.experts
+    if args.moe_step:
+        cfg["interleave_moe_layer_step"] = args.moe_step
     item = 2 if args.dtype == "bf16" else 4
     points = [int(x) for x in args.points.split(",") if x.strip()]
     max_b = max([args.batch] + points)
@@ -204,7 +218,8 @@ def main() -> int:
         "config": {"model": "llama4-scout-shape" if not args.tiny else "llama4-tiny-shape", "layers": L,
                    "layers_full": layers_full, "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
                    "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
-                   "experts": cfg["num_local_experts"], "top_k": 1, "expert_intermediate": cfg["intermediate_size"],
+                   "experts": cfg["num_local_experts"], "moe_every": cfg["interleave_moe_layer_step"], "top_k": 1,
+                   "expert_intermediate": cfg["intermediate_size"],
                    "shared_expert": 1, "vocab": V, "chunk": cfg["attention_chunk_size"], "nope_every": 4,
                    "global_batch": args.batch, "seq_len": args.context, "page_size": page,
                    "parallelism": "none (1 GPU)"},
