@@ -65,6 +65,38 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+// Which group and which rows the row tile `mt` of a grouped product covers.  Groups are walked
+// in order, group e bringing ceil((offsets[e+1] - offsets[e]) / MT) tiles of MT rows.  A wave
+// looks at 64 groups at a time (a prefix sum over its lanes), so that hundreds of groups cost a
+// few steps; every lane of the wave must call it and gets the same answer.  False: mt lies
+// past the last tile.
+__device__ __forceinline__ bool sp_find_tile(const int* offsets, int n_groups, int MT, int mt,
+                                             int& g, int& row0, int& row_end) {
+    const int lane = threadIdx.x & 63;
+    int base = 0;
+    for (int c = 0; c < n_groups; c += 64) {
+        const int e = c + lane;
+        int b = 0, en = 0;
+        if (e < n_groups) { b = offsets[e]; en = offsets[e + 1]; }
+        const int nt = (en - b + MT - 1) / MT;
+        int incl = nt;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) { const int v = __shfl_up(incl, o, 64); if (lane >= o) incl += v; }
+        const int total = __shfl(incl, 63, 64);
+        if (mt < base + total) {
+            const bool mine = mt >= base + incl - nt && mt < base + incl;
+            const int src = __ffsll((unsigned long long)__ballot(mine)) - 1;
+            // the same in every lane: say so, to keep them in scalar registers
+            g = __builtin_amdgcn_readfirstlane(c + src);
+            row0 = __builtin_amdgcn_readfirstlane(__shfl(b, src, 64) + (mt - base - __shfl(incl - nt, src, 64)) * MT);
+            row_end = __builtin_amdgcn_readfirstlane(__shfl(en, src, 64));
+            return true;
+        }
+        base += total;
+    }
+    return false;
+}
+
 // Sum over a workgroup of NT threads (NT a multiple of 64, at most 1024); every thread
 // gets the result.  `red` is shared scratch of at least NT/64 floats; two barriers.
 template <int NT>

@@ -26,15 +26,7 @@ void gemm_generic_kernel(const T* __restrict__ A, int lda, const T* __restrict__
     // ---- which group and which of its row tiles
     int g = 0, row0 = 0, row_end = M;
     if (offsets) {
-        int mt = blockIdx.y, acc = 0;
-        g = -1;
-        for (int e = 0; e < n_groups; ++e) {
-            const int b = offsets[e], en = offsets[e + 1];
-            const int nt = (en - b + GBM - 1) / GBM;
-            if (mt < acc + nt) { g = e; row0 = b + (mt - acc) * GBM; row_end = en; break; }
-            acc += nt;
-        }
-        if (g < 0) return;
+        if (!sp_find_tile(offsets, n_groups, GBM, blockIdx.y, g, row0, row_end)) return;
     } else {
         row0 = blockIdx.y * GBM;
         if (row0 >= M) return;

@@ -38,15 +38,7 @@ void gemm_skinny_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restr
 
     int g = 0, row0, row_end = M;
     if (offsets) {
-        int mt = blockIdx.y, acc = 0;
-        g = -1;
-        for (int e = 0; e < n_groups; ++e) {
-            const int b = offsets[e], en = offsets[e + 1];
-            const int nt = (en - b + MT - 1) / MT;
-            if (mt < acc + nt) { g = e; row0 = b + (mt - acc) * MT; row_end = en; break; }
-            acc += nt;
-        }
-        if (g < 0) return;
+        if (!sp_find_tile(offsets, n_groups, MT, blockIdx.y, g, row0, row_end)) return;
     } else {
         row0 = blockIdx.y * MT;
         if (row0 >= M) return;
@@ -212,7 +204,8 @@ extern "C" int spite_gemm_skinny(const void* X, int ldx, const void* W, long w_g
             else if ((size_t)N * K >= ((size_t)1 << 28)) variant = max_rows <= 8 ? 4 : 7;
             else variant = 8;
         }
-        else variant = max_rows <= 32 ? 2 : (offsets && !glu ? 3 : 9);
+        else if (max_rows <= 32) variant = !offsets && (size_t)N * K >= ((size_t)1 << 28) ? 10 : 2;
+        else variant = offsets && !glu ? 3 : 9;
     }
     switch (variant) {
         case 1: return launch_skinny<1, 1, 4, 8>(SP_ARGS);
@@ -224,6 +217,7 @@ extern "C" int spite_gemm_skinny(const void* X, int ldx, const void* W, long w_g
         case 7: return launch_skinny<4, 1, 2, 8>(SP_ARGS);
         case 8: return launch_skinny<2, 1, 2, 8>(SP_ARGS);
         case 9: return launch_skinny<2, 4, 2, 8>(SP_ARGS);
+        case 10: return launch_skinny<4, 2, 2, 8>(SP_ARGS);
         default: return sp_fail("gemm_skinny: unknown variant %d", variant);
     }
 #undef SP_ARGS

@@ -44,15 +44,7 @@ void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restri
     const int tile_m = tile_id % m_tiles, tile_n = tile_id / m_tiles;
     int g = 0, row0, row_end = M;
     if (offsets) {
-        int mt = tile_m, acc = 0;
-        g = -1;
-        for (int e = 0; e < n_groups; ++e) {
-            const int b = offsets[e], en = offsets[e + 1];
-            const int nt = (en - b + BM - 1) / BM;
-            if (mt < acc + nt) { g = e; row0 = b + (mt - acc) * BM; row_end = en; break; }
-            acc += nt;
-        }
-        if (g < 0) return;
+        if (!sp_find_tile(offsets, n_groups, BM, tile_m, g, row0, row_end)) return;
     } else {
         row0 = tile_m * BM;
         if (row0 >= M) return;

@@ -148,8 +148,8 @@ def gemm_reference(a, w, M, N, K, offsets=None, a_rows=None, a_scale=None, y_row
 GEMM_SHAPES = [(1, 48, 64), (7, 100, 264), (16, 130, 1032), (33, 96, 96), (64, 72, 520), (5, 202, 144)]
 
 
-def run_gemm(fn, dtype, out_dtype, M, N, K, glu=False, grouped=False, **kw):
-    E = 5 if grouped else 1
+def run_gemm(fn, dtype, out_dtype, M, N, K, glu=False, grouped=False, groups=5, **kw):
+    E = groups if grouped else 1
     a = rnd(M + 3, K, dtype=dtype, scale=0.5)
     w = rnd(*((E,) if grouped else ()), (2 * N if glu else N), K, dtype=dtype, seed=1, scale=0.5)
     args = dict(glu=glu)
@@ -185,7 +185,7 @@ def test_gemm_generic(M, N, K, dtype, out_dtype, glu, grouped):
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES + [(3, 40, 8), (12, 16, 4104)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("glu,grouped", [(False, False), (True, False), (False, True), (True, True)])
-@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8, 9])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10])
 def test_gemm_skinny(M, N, K, out_dtype, glu, grouped, variant):
     run_gemm(ops().gemm_skinny, torch.bfloat16, out_dtype, M, N, K, glu, grouped, variant=variant)
 
@@ -204,7 +204,7 @@ TILED_SHAPES = [(1, 48, 64), (7, 112, 320), (16, 144, 1088), (64, 80, 512), (33,
 @pytest.mark.parametrize("M,N,K", TILED_SHAPES)
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("glu,grouped", [(False, False), (True, False), (False, True), (True, True)])
-@pytest.mark.parametrize("variant", [2, 3, 4, 6, 7, 8, 9])
+@pytest.mark.parametrize("variant", [2, 3, 4, 6, 7, 8, 9, 10])
 def test_gemm_skinny_over_operand_order(M, N, K, out_dtype, glu, grouped, variant):
     def fn(a, w, y, *args, **kw):
         ops().gemm_skinny(a, ops().operand_order(w), y, *args, tiled=True, **kw)
@@ -220,6 +220,26 @@ def test_gemm_tiled(M, N, K, out_dtype, glu, grouped, shape):
     def fn(a, w, y, *args, **kw):
         ops().gemm_tiled(a, ops().operand_order(w), y, *args, **kw)
     run_gemm(fn, torch.bfloat16, out_dtype, M, N, K, glu, grouped, shape=shape)
+
+
+@pytest.mark.parametrize("M,groups", [(40, 150), (300, 150), (9, 64), (70, 65), (500, 129)])
+@pytest.mark.parametrize("glu", [False, True])
+def test_gemm_over_many_groups(M, groups, glu):
+    """More groups than a wave has lanes, most of them empty or with a row or two: the search
+    for a row tile's group walks them 64 at a time."""
+    N, K = 48, 128
+    run_gemm(ops().gemm_generic, torch.float32, torch.float32, M, N, K, glu, True, groups=groups)
+    run_gemm(ops().gemm_mfma, torch.bfloat16, torch.float32, M, N, K, glu, True, groups=groups)
+
+    def tiled(a, w, y, *args, **kw):
+        ops().gemm_tiled(a, ops().operand_order(w), y, *args, **kw)
+    run_gemm(tiled, torch.bfloat16, torch.float32, M, N, K, glu, True, groups=groups)
+    if M <= 64:
+        for variant in (2, 8, 9):
+            def skinny(a, w, y, *args, **kw):
+                ops().gemm_skinny(a, ops().operand_order(w), y, *args, tiled=True, variant=variant, **kw)
+            run_gemm(skinny, torch.bfloat16, torch.float32, M, N, K, glu, True, groups=groups)
+            run_gemm(ops().gemm_skinny, torch.bfloat16, torch.float32, M, N, K, glu, True, groups=groups, variant=variant)
 
 
 def test_gemm_tiled_refuses_what_it_cannot_do():
