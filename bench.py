@@ -68,7 +68,15 @@ def decode_bytes(cfg, L, batch, context, experts_touched, item=2):
         + batch * seen * kv_token + V * d * item + batch * d * item + d * 4
 
 
-def prefill_flops(cfg, L, T):
+def visible_pairs(T, past, span=None):
+    """(query, key) pairs of a portion of T tokens that follows `past` cached ones: every key up
+    to the query itself, or only those of the query's own chunk of `span` positions."""
+    if span is None:
+        return T * past + T * (T + 1) // 2
+    return sum(p % span + 1 for p in range(past, past + T))
+
+
+def prefill_flops(cfg, L, T, past=0):
     d, H, G, hd = cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
     F, V = cfg["intermediate_size"], cfg["vocab_size"]
     step = cfg["interleave_moe_layer_step"]
@@ -76,8 +84,9 @@ def prefill_flops(cfg, L, T):
     proj = (H + 2 * G) * hd * d + d * H * hd
     moe = 2 * 3 * d * F + cfg["num_local_experts"] * d            # one routed expert and the shared one a token
     dense = 3 * d * cfg["intermediate_size_mlp"]
-    attn = 4 * (T * (T + 1) // 2) * H * hd
-    return L * (2 * proj * T + attn) + 2 * T * (n_moe * moe + (L - n_moe) * dense) + 2 * d * V
+    n_full = sum(1 for layer in range(L) if (layer + 1) % 4 == 0)
+    pairs = n_full * visible_pairs(T, past) + (L - n_full) * visible_pairs(T, past, cfg["attention_chunk_size"])
+    return L * 2 * proj * T + 4 * pairs * H * hd + 2 * T * (n_moe * moe + (L - n_moe) * dense) + 2 * d * V
 
 
 def main() -> int:
@@ -89,6 +98,8 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--prefill-context", type=int, default=0,
+                    help="the timed prompt portion follows this many tokens already in the cache")
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--tiny", action="store_true", help="a small model of the same kind, to try the script")
@@ -121,7 +132,7 @@ def main() -> int:
     max_b = max([args.batch] + points)
     page = 64
     per_req = -(-(args.context + args.steps + args.warmup + 8) // page) * page
-    cache_tokens = max(max_b * per_req, args.prefill_tokens + page)
+    cache_tokens = max(max_b * per_req, args.prefill_context + args.prefill_tokens + 2 * page)
     log(f"building {L} of {layers_full} layers, cache for {cache_tokens} positions")
     t0 = time.time()
     eng = Engine(cfg, dtype=args.dtype, page_size=page, cache_tokens=cache_tokens, max_requests=max_b,
@@ -137,6 +148,9 @@ def main() -> int:
     # ---- prefill of one prompt
     def prefill_once():
         s = eng.admit()
+        if args.prefill_context:
+            eng.cache.reserve(s, args.prefill_context)
+            eng.cache.commit(s, args.prefill_context)
         toks = rng.randint(0, V, size=args.prefill_tokens).tolist()
         torch.cuda.synchronize()
         t = time.perf_counter()
@@ -148,12 +162,18 @@ def main() -> int:
         return dt
     prefill = None
     if args.phase != "decode":
+        if args.prefill_context:
+            for g in eng.cache.groups:
+                g.kv.normal_(0.0, 1.0)
         prefill_once()
         pre = min(prefill_once() for _ in range(2))
-        pf = prefill_flops(cfg, L, args.prefill_tokens)
+        pf = prefill_flops(cfg, L, args.prefill_tokens, args.prefill_context)
         prefill = {"value": round(args.prefill_tokens / pre, 1), "tokens": args.prefill_tokens,
                    "ms": round(pre * 1e3, 3), "frac": round(pf / pre / MFMA_PEAK[args.dtype], 4)}
-        log(f"prefill {args.prefill_tokens} tokens: {pre * 1e3:.1f} ms")
+        if args.prefill_context:
+            prefill["after"] = args.prefill_context
+        log(f"prefill {args.prefill_tokens} tokens" + (f" after {args.prefill_context}" if args.prefill_context else "")
+            + f": {pre * 1e3:.1f} ms")
     if args.phase == "prefill":
         print(json.dumps({"metric": "prefill only", "value": None, "prefill": prefill, "n_gpus": 1,
                           "config": {"layers": L, "layers_full": layers_full}}))

@@ -10,10 +10,11 @@
 // that path, not the MFMA units or LDS, is what bounds this kernel.  The tiles of one row
 // band follow each other in k, so a wave streams its four bands.
 //
-// A workgroup of eight waves owns 128*WM rows of X ("slots") and 64*WN rows of W
-// (WN * WM = 8); a wave owns 64 rows of W and 128 slots: 4 x 8 accumulator tiles.
+// A workgroup of eight waves owns 16*NB*WM rows of X ("slots") and 64*WN rows of W
+// (WN * WM = 8); a wave owns 64 rows of W and 16*NB slots: 4 x NB accumulator tiles (NB = 8,
+// or 10 where the registers of the third W set go to the accumulators).
 //  * W never touches LDS: three rotating sets of operand registers, loaded two steps of 32 k
-//    ahead of the products.
+//    ahead of the products (NB = 10: two sets, one step ahead).
 //  * X is the "B" operand, shared by the waves: tiles of 64 k go through LDS, fetched with
 //    eight lanes a row (whole cache lines), rows padded by 16 bytes against bank conflicts,
 //    double-buffered, one barrier per 64 k.
@@ -25,14 +26,15 @@
 
 #define TLD 72             // padded row of the X tile in LDS, in elements (64 k + 8)
 
-template <int WN, int WM, bool GLU, typename TY>
+template <int WN, int WM, int NB, bool GLU, typename TY>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restrict__ W, long w_group_stride,
                        TY* __restrict__ Y, int ldy, int M, int N, int K,
                        const int* __restrict__ offsets, int n_groups, const int* __restrict__ a_rows,
                        const float* __restrict__ a_scale, const int* __restrict__ y_rows, int m_tiles, int n_tiles) {
     static_assert(WN * WM == 8, "eight waves");
-    constexpr int BM = 128 * WM, BN = 64 * WN;
+    constexpr int WS = 16 * NB;                     // slots of a wave: NB slot tiles
+    constexpr int BM = WS * WM, BN = 64 * WN;
     constexpr int NCOLS = GLU ? BN / 2 : BN;        // output columns per workgroup
     extern __shared__ __attribute__((aligned(16))) bf16 Xs[];     // [2][BM * TLD]
 
@@ -56,7 +58,7 @@ void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restri
     const int r = lane & 15, q = lane >> 4;
 
     // ---- X: global -> registers -> LDS; thread loads 16-byte chunk (tid % 8) of rows tid/8 + 64*i
-    constexpr int XL = 2 * WM;
+    constexpr int XL = (BM + 63) / 64;
     const int lrow = tid >> 3, lchunk = tid & 7;
     const bf16* xsrc[XL];
 #pragma unroll
@@ -86,11 +88,14 @@ void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restri
     auto load_x = [&](bf16x8 (&xr)[XL], int u) {
         const int k0 = (u < nu ? u : nu - 1) * 64;
 #pragma unroll
-        for (int i = 0; i < XL; ++i) xr[i] = *(const bf16x8*)(xsrc[i] + k0);
+        for (int i = 0; i < XL; ++i)
+            if (64 * (i + 1) <= BM || lrow + 64 * i < BM) xr[i] = *(const bf16x8*)(xsrc[i] + k0);   // (whole waves)
     };
     auto store_x = [&](bf16x8 (&xr)[XL], int buf) {
 #pragma unroll
-        for (int i = 0; i < XL; ++i) *(bf16x8*)(Xs + buf * (BM * TLD) + (lrow + 64 * i) * TLD + lchunk * 8) = xr[i];
+        for (int i = 0; i < XL; ++i)
+            if (64 * (i + 1) <= BM || lrow + 64 * i < BM)
+                *(bf16x8*)(Xs + buf * (BM * TLD) + (lrow + 64 * i) * TLD + lchunk * 8) = xr[i];
     };
     auto load_w = [&](bf16x8 (&ws)[4], int t) {
         const size_t at = (size_t)(t < kt ? t : kt - 1) * 512;
@@ -98,23 +103,26 @@ void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restri
         for (int a = 0; a < 4; ++a) ws[a] = *(const bf16x8*)(wsrc[a] + at);
     };
 
-    f32x4 acc[4][8];           // [W band a][slot tile b]
+    f32x4 acc[4][NB];          // [W band a][slot tile b]
 #pragma unroll
     for (int a = 0; a < 4; ++a)
 #pragma unroll
-        for (int b = 0; b < 8; ++b) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int b = 0; b < NB; ++b) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
     auto mul = [&](bf16x8 (&ws)[4], int buf, int kk) {
-        const bf16* xs = Xs + buf * (BM * TLD) + (wm * 128 + r) * TLD + kk * 32 + q * 8;
+        const bf16* xs = Xs + buf * (BM * TLD) + (wm * WS + r) * TLD + kk * 32 + q * 8;
+        constexpr int NX = 4;                        // slot tiles read from LDS at a time
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            bf16x8 xf[4];
+        for (int b0 = 0; b0 < NB; b0 += NX) {
+            bf16x8 xf[NX];
 #pragma unroll
-            for (int b = 0; b < 4; ++b) xf[b] = *(const bf16x8*)(xs + (half * 4 + b) * 16 * TLD);
+            for (int b = 0; b < NX; ++b)
+                if (b0 + b < NB) xf[b] = *(const bf16x8*)(xs + (b0 + b) * 16 * TLD);
 #pragma unroll
             for (int a = 0; a < 4; ++a)
 #pragma unroll
-                for (int b = 0; b < 4; ++b)
-                    acc[a][half * 4 + b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ws[a], xf[b], acc[a][half * 4 + b], 0, 0, 0);
+                for (int b = 0; b < NX; ++b)
+                    if (b0 + b < NB)
+                        acc[a][b0 + b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ws[a], xf[b], acc[a][b0 + b], 0, 0, 0);
         }
     };
 
@@ -137,26 +145,47 @@ void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restri
         store_x(xr, (u + 1) & 1);
         __syncthreads();
     };
-    load_x(xr, 0);
-    load_w(w0, 0);
-    load_w(w1, 1);
-    store_x(xr, 0);
-    __syncthreads();
-    int u = 0;
-    for (; u + 3 <= nu; u += 3) {
-        step(w0, w1, w2, u);            // half steps 0, 1: use w0, w1; load w2 (t=2), w0 (t=3)
-        step(w2, w0, w1, u + 1);        // half steps 2, 3: use w2, w0; load w1 (t=4), w2 (t=5)
-        step(w1, w2, w0, u + 2);        // half steps 4, 5: use w1, w2; load w0 (t=6), w1 (t=7)
-    }
-    if (u < nu) {
-        step(w0, w1, w2, u);
-        if (u + 1 < nu) step(w2, w0, w1, u + 1);
+    if constexpr (NB == 8) {
+        load_x(xr, 0);
+        load_w(w0, 0);
+        load_w(w1, 1);
+        store_x(xr, 0);
+        __syncthreads();
+        int u = 0;
+        for (; u + 3 <= nu; u += 3) {
+            step(w0, w1, w2, u);            // half steps 0, 1: use w0, w1; load w2 (t=2), w0 (t=3)
+            step(w2, w0, w1, u + 1);        // half steps 2, 3: use w2, w0; load w1 (t=4), w2 (t=5)
+            step(w1, w2, w0, u + 2);        // half steps 4, 5: use w1, w2; load w0 (t=6), w1 (t=7)
+        }
+        if (u < nu) {
+            step(w0, w1, w2, u);
+            if (u + 1 < nu) step(w2, w0, w1, u + 1);
+        }
+    } else {
+        // more slot tiles a wave: the registers of the third set go to the accumulators, and a
+        // set is asked for again as soon as its products are issued, one half step ahead
+        load_x(xr, 0);
+        load_w(w0, 0);
+        load_w(w1, 1);
+        store_x(xr, 0);
+        __syncthreads();
+        for (int u = 0; u < nu; ++u) {
+            load_x(xr, u + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            mul(w0, u & 1, 0);
+            load_w(w0, 2 * u + 2);
+            __builtin_amdgcn_sched_barrier(0);
+            mul(w1, u & 1, 1);
+            load_w(w1, 2 * u + 3);
+            store_x(xr, (u + 1) & 1);
+            __syncthreads();
+        }
     }
 
-    // acc[a][b][i] of lane (r, q): column ncol[a] + q*4 + i, slot row0 + wm*128 + b*16 + r
+    // acc[a][b][i] of lane (r, q): column ncol[a] + q*4 + i, slot row0 + wm*WS + b*16 + r
 #pragma unroll
-    for (int b = 0; b < 8; ++b) {
-        const int s = row0 + wm * 128 + b * 16 + r;
+    for (int b = 0; b < NB; ++b) {
+        const int s = row0 + wm * WS + b * 16 + r;
         if (s >= row_end) continue;
         const float sc = a_scale ? a_scale[s] : 1.0f;
         const size_t yr = y_rows ? (size_t)y_rows[s] : (size_t)s;
@@ -185,11 +214,11 @@ void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restri
     }
 }
 
-template <int WN, int WM, bool GLU, typename TY>
+template <int WN, int WM, int NB, bool GLU, typename TY>
 static int launch_tiled_kernel(const void* X, int ldx, const void* W, long w_group_stride, void* Y, int ldy, int M, int N,
                                int K, const int* offsets, int n_groups, const int* a_rows, const float* a_scale,
                                const int* y_rows, hipStream_t st) {
-    constexpr int BM = 128 * WM, BN = 64 * WN;
+    constexpr int BM = 16 * NB * WM, BN = 64 * WN;
     const int m_tiles = (M + BM - 1) / BM + (offsets ? n_groups : 0);
     const int ncols = GLU ? BN / 2 : BN;
     const int n_tiles = (N + ncols - 1) / ncols;
@@ -197,23 +226,23 @@ static int launch_tiled_kernel(const void* X, int ldx, const void* W, long w_gro
     const size_t sh = (size_t)2 * BM * TLD * sizeof(bf16);
     static bool allowed = false;        // one flag per instantiation; more LDS than the default limit for WM = 2
     if (!allowed) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<WN, WM, GLU, TY>,
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<WN, WM, NB, GLU, TY>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)sh);
         SP_REQUIRE(e == hipSuccess, "gemm_tiled: %zu bytes of LDS refused: %s", sh, hipGetErrorString(e));
         allowed = true;
     }
-    gemm_tiled_kernel<WN, WM, GLU, TY><<<dim3((m_tiles * n_tiles + 7) / 8 * 8), 512, sh, st>>>(
+    gemm_tiled_kernel<WN, WM, NB, GLU, TY><<<dim3((m_tiles * n_tiles + 7) / 8 * 8), 512, sh, st>>>(
         (const bf16*)X, ldx, (const bf16*)W, w_group_stride, (TY*)Y, ldy, M, N, K, offsets, n_groups, a_rows, a_scale,
         y_rows, m_tiles, n_tiles);
     SP_LAUNCH_CHECK("gemm_tiled");
     return 0;
 }
 
-template <int WN, int WM>
+template <int WN, int WM, int NB>
 static int launch_tiled(const void* X, int ldx, const void* W, long w_group_stride, void* Y, int y_dtype, int ldy, int M,
                         int N, int K, const int* offsets, int n_groups, const int* a_rows, const float* a_scale,
                         const int* y_rows, int glu, hipStream_t st) {
-#define SP_TL(GLUV, TY) launch_tiled_kernel<WN, WM, GLUV, TY>(X, ldx, W, w_group_stride, Y, ldy, M, N, K, offsets, n_groups, \
+#define SP_TL(GLUV, TY) launch_tiled_kernel<WN, WM, NB, GLUV, TY>(X, ldx, W, w_group_stride, Y, ldy, M, N, K, offsets, n_groups, \
                                                               a_rows, a_scale, y_rows, st)
     if (glu) return y_dtype == SP_BF16 ? SP_TL(true, bf16) : SP_TL(true, float);
     return y_dtype == SP_BF16 ? SP_TL(false, bf16) : SP_TL(false, float);
@@ -221,7 +250,8 @@ static int launch_tiled(const void* X, int ldx, const void* W, long w_group_stri
 }
 
 // W in operand order (see above), every group N (2N with GLU) rows of K.
-// `shape`: 0 lets the library choose; 1 = 512 W rows x 128 slots a workgroup, 2 = 256 x 256.
+// `shape`: 0 lets the library choose; 1 = 512 W rows x 128 slots a workgroup, 2 = 256 x 256,
+// 3 = 512 x 160 (for groups of a little over 128 rows, which would need a second tile of 128).
 extern "C" int spite_gemm_tiled(const void* X, int ldx, const void* W, long w_group_stride, void* Y, int y_dtype,
                                 int ldy, int M, int N, int K, const int* offsets, int n_groups, const int* a_rows,
                                 const float* a_scale, const int* y_rows, int glu, int shape, hipStream_t st) {
@@ -231,10 +261,12 @@ extern "C" int spite_gemm_tiled(const void* X, int ldx, const void* W, long w_gr
     SP_REQUIRE(((uintptr_t)X & 15) == 0 && ((uintptr_t)W & 15) == 0, "gemm_tiled: operands must be 16-byte aligned");
     SP_REQUIRE(y_dtype == SP_BF16 || y_dtype == SP_F32, "gemm_tiled: output dtype %d", y_dtype);
     SP_REQUIRE(!offsets || n_groups > 0, "gemm_tiled: grouped call without groups");
-    SP_REQUIRE(shape >= 0 && shape <= 2, "gemm_tiled: tile shape %d", shape);
+    SP_REQUIRE(shape >= 0 && shape <= 3, "gemm_tiled: tile shape %d", shape);
     if (M == 0) return 0;
     if (shape == 0) shape = 1;          // measured the faster one at every shape of Llama 4 Scout
     if (shape == 1)
-        return launch_tiled<8, 1>(X, ldx, W, w_group_stride, Y, y_dtype, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, st);
-    return launch_tiled<4, 2>(X, ldx, W, w_group_stride, Y, y_dtype, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, st);
+        return launch_tiled<8, 1, 8>(X, ldx, W, w_group_stride, Y, y_dtype, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, st);
+    if (shape == 3)
+        return launch_tiled<8, 1, 10>(X, ldx, W, w_group_stride, Y, y_dtype, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, st);
+    return launch_tiled<4, 2, 8>(X, ldx, W, w_group_stride, Y, y_dtype, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, st);
 }

@@ -14,7 +14,7 @@ from __future__ import annotations
 import torch
 
 from .base import FeedForward, ParamSpec, register
-from .linear import linear, Weight
+from .linear import SKINNY_MAX_ROWS, Weight, grouped_tile_shape, linear
 from ..csrc import hipops
 
 
@@ -104,10 +104,12 @@ class MoeTop1Sigmoid(FeedForward):
         if ctx.extras.get("trace") is not None:      # a testing aid: which expert each row took
             ctx.extras["trace"].setdefault("moe_experts", []).append(expert.clone())
         act = ws.take((n, F), x.dtype)
+        shape = grouped_tile_shape(T, E, groups - E) if T > SKINNY_MAX_ROWS else 0
         linear(x, self.w_gate_up, act, glu=True, offsets=offsets, n_groups=groups, a_rows=src, a_scale=scale, rows=n,
-               max_rows=T)
+               max_rows=T, tile_shape=shape)
         # slot s writes row dst[s]: rows [0,T) the routed result per token, rows [T,2T) the shared one
         y = ws.take((2 * T, d), torch.float32)
+        # (the down product has too few column tiles for the larger row tile to pay)
         linear(act, self.w_down, y, offsets=offsets, n_groups=groups, y_rows=dst, rows=n, max_rows=T)
         if self.fused_shared:
             return (y[:T], y[T:])

@@ -6,6 +6,8 @@
 """
 from __future__ import annotations
 
+import math
+
 import torch
 
 from ..csrc import hipops
@@ -36,12 +38,34 @@ class Weight:
         self.data = hipops.operand_order(w) if self.tiled else w
 
 
+def grouped_tile_shape(tokens: int, groups: int, whole_groups: int = 0) -> int:
+    """Which tile of the prefill product suits ``tokens`` rows that spread evenly over ``groups``
+    groups (experts that a router picks), beside ``whole_groups`` groups that take every row.
+    A group costs whole row tiles, each of which streams the group's weights once: with 128
+    rows a tile (shape 1) half of the groups of about 128 rows need a second tile, with 160
+    (shape 3, about a sixth dearer per tile) almost none.  The expected number of tiles of
+    each shape decides, group sizes taken as normal around tokens/groups."""
+    if groups <= 0 or tokens <= 0:
+        return 1
+    mean = tokens / groups
+    sd = max(math.sqrt(tokens * (1.0 / groups) * (1.0 - 1.0 / groups)), 1e-6)
+
+    def tiles(rows_per_tile):
+        extra, k = 0.0, 1
+        while k * rows_per_tile < mean + 6 * sd:
+            extra += 0.5 * math.erfc((k * rows_per_tile + 0.5 - mean) / (sd * math.sqrt(2.0)))
+            k += 1
+        return groups * (1.0 + extra) + whole_groups * -(-tokens // rows_per_tile)
+    return 3 if 1.17 * tiles(160) < tiles(128) else 1
+
+
 def linear(x, w, y, *, glu=False, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None, rows=None,
-           max_rows=None):
+           max_rows=None, tile_shape=0):
     """y[r] = W . x[r] for ``rows`` rows (default: all of x; for a row list: its length).
 
     With ``glu`` the weight holds gate rows then up rows and y = silu(gate) * up.
-    ``max_rows``: the most rows that one group can bring (default: ``rows``)."""
+    ``max_rows``: the most rows that one group can bring (default: ``rows``).
+    ``tile_shape``: the prefill product's tile (``grouped_tile_shape``), 0 = the library's choice."""
     tiled = False
     if isinstance(w, Weight):
         w, tiled = w.data, w.tiled
@@ -57,7 +81,7 @@ def linear(x, w, y, *, glu=False, offsets=None, n_groups=1, a_rows=None, a_scale
                                a_scale=a_scale, y_rows=y_rows, glu=glu, max_rows=most, tiled=tiled)
         elif tiled:
             hipops.gemm_tiled(x, w, y, M, N, K, offsets=offsets, n_groups=n_groups, a_rows=a_rows, a_scale=a_scale,
-                              y_rows=y_rows, glu=glu)
+                              y_rows=y_rows, glu=glu, shape=tile_shape)
         else:
             hipops.gemm_mfma(x, w, y, M, N, K, offsets=offsets, n_groups=n_groups, a_rows=a_rows, a_scale=a_scale,
                              y_rows=y_rows, glu=glu)
