@@ -42,6 +42,7 @@ def lib():
             "spite_gemm_generic": [P, I, P, L, I, P, I, I, I, I, I, P, I, P, P, P, I, P],
             "spite_attn_generic": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, I, P],
             "spite_sample_rows": [P, I, I, I, P, P, P, P],
+            "spite_filter_rows": [P, I, I, I, P, P, P, P],
             "spite_gemm_skinny": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, I, I, P],
             "spite_attn_decode": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, P],
             "spite_gemm_mfma": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, P],
@@ -262,6 +263,21 @@ def sample_rows(logits, temperature, uniform, out, n_rows=None):
                                    _ptr(temperature, "temperature", torch.float32, True),
                                    _ptr(uniform, "uniform", torch.float32, True),
                                    _ptr(out, "out", torch.int32), _stream()), "sample")
+
+
+def filter_rows(work, params, pen_ids, pen_offsets):
+    """The reference's filters on the rows of ``work`` (fp32 [n, V]) in place: repetition
+    penalty, temperature, min-p, top-k, top-p (see sampling.hip).  ``params``: float64 [6, n]
+    (on, temperature, ln(min_p), top_k, top_p, penalty); ``pen_ids`` int32, row r's distinct ids
+    at ``pen_offsets[r] .. pen_offsets[r+1]`` (int32 [n+1]); the caller keeps the ids inside [0, V)."""
+    n = work.shape[0]
+    if params.dtype != torch.float64 or tuple(params.shape) != (6, n) or not params.is_contiguous():
+        raise KernelError(f"filter: params {tuple(params.shape)} {params.dtype} for {n} rows")
+    if pen_offsets.numel() != n + 1:
+        raise KernelError(f"filter: {pen_offsets.numel()} offsets for {n} rows")
+    _check(lib().spite_filter_rows(_ptr(work, "work", torch.float32), work.stride(0), n, work.shape[1],
+                                   _ptr(params, "params", torch.float64), _ptr(pen_ids, "pen_ids", torch.int32, True),
+                                   _ptr(pen_offsets, "pen_offsets", torch.int32), _stream()), "filter")
 
 
 def _gemm_checks(a, w, y, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, what):

@@ -3,7 +3,8 @@
 distinct id once) -> /temperature -> min-p -> top-k -> top-p -> greedy when temperature <= 0,
 else the inverse-CDF draw with one LCG stream per request (:343-348).  Names and meanings of
 the options are the reference's ``SamplerConfig`` (:83-111); the defaults here switch every
-filter off.  Greedy takes the lowest index among equal maxima.
+filter off.  Greedy takes the lowest index among equal maxima.  The filters of all rows of a
+step run in one kernel (``filter_rows``), the draws in another; the host only packs the options.
 """
 from __future__ import annotations
 
@@ -47,32 +48,25 @@ class Sampler:
         self.device = device
         self._scratch = None
 
-    def _process_row(self, row: torch.Tensor, p: SamplingParams, context: Sequence[int]) -> torch.Tensor:
-        l = row.clone()
-        V = l.numel()
-        if abs(p.repetition_penalty - 1.0) >= 1.1920929e-07 and len(context):
-            win = context if p.repeat_last_n == 0 or p.repeat_last_n >= len(context) else context[-p.repeat_last_n:]
-            ids = sorted({int(t) for t in win if 0 <= int(t) < V})
-            if ids:
-                idx = torch.tensor(ids, dtype=torch.long, device=l.device)
-                v = l[idx]
-                l[idx] = torch.where(v > 0, v / p.repetition_penalty, v * p.repetition_penalty)
-        if p.temperature > 0:
-            l = l / p.temperature
-        if p.min_p > 0:
-            l = l.masked_fill(l < l.max() + math.log(p.min_p), float("-inf"))
-        if 0 < p.top_k < V:
-            thresh = torch.topk(l, p.top_k).values[-1]
-            l = l.masked_fill(l < thresh, float("-inf"))
-        if p.top_p < 1.0:
-            vals, order = torch.sort(l, descending=True, stable=True)
-            e = torch.exp(vals - vals[0])
-            total = e.sum()
-            cum = torch.cumsum(e, 0) / total
-            reached = (cum >= p.top_p).nonzero()
-            kept = int(reached[0]) + 1 if reached.numel() else V
-            l[order[max(kept, 1):]] = float("-inf")
-        return l
+    def _filter(self, work: torch.Tensor, params: Sequence[SamplingParams], contexts: Sequence[Sequence[int]]):
+        """Runs the filters of the rows that ask for them over ``work`` in place (one kernel)."""
+        n, V = work.shape
+        table = np.zeros((6, n), dtype=np.float64)
+        ids: List[int] = []
+        offsets = np.zeros(n + 1, dtype=np.int32)
+        for i, p in enumerate(params):
+            if p.filters():
+                table[:, i] = (1.0, max(p.temperature, 0.0), math.log(p.min_p) if p.min_p > 0 else -math.inf,
+                               p.top_k if 0 < p.top_k < V else 0, p.top_p, p.repetition_penalty)
+                context = contexts[i]
+                if abs(p.repetition_penalty - 1.0) >= 1.1920929e-07 and len(context):
+                    win = (context if p.repeat_last_n == 0 or p.repeat_last_n >= len(context)
+                           else context[-p.repeat_last_n:])
+                    ids.extend(sorted({int(t) for t in win if 0 <= int(t) < V}))
+            offsets[i + 1] = len(ids)
+        dev = work.device
+        pen_ids = torch.tensor(ids, dtype=torch.int32, device=dev) if ids else None
+        hipops.filter_rows(work, torch.from_numpy(table).to(dev), pen_ids, torch.from_numpy(offsets).to(dev))
 
     def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], contexts: Sequence[Sequence[int]],
                rng_states: List[int]) -> List[int]:
@@ -86,9 +80,7 @@ class Sampler:
         work = logits
         if any(p.filters() for p in params):
             work = logits.clone()
-            for i, p in enumerate(params):
-                if p.filters():
-                    work[i] = self._process_row(logits[i], p, contexts[i])
+            self._filter(work, params, contexts)
         for i, p in enumerate(params):
             if p.temperature > 0:
                 temps[i] = 1.0 if p.filters() else p.temperature     # filtered rows are divided already

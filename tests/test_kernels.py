@@ -599,3 +599,58 @@ def test_argmax_and_sampling_rows(V):
     masked[:, 1:] = float("-inf")
     ops().sample_rows(masked, torch.ones(n, device=DEV), torch.rand(n, device=DEV), out)
     assert out.cpu().tolist() == [0] * n
+
+
+def _filter_case(row, ctx, temperature=0.0, top_k=0, top_p=1.0, min_p=0.0, penalty=1.0, last_n=0):
+    l = plain.apply_repetition_penalty(row.clone(), ctx, penalty, last_n)
+    l = plain.apply_temperature(l, temperature)
+    l = plain.apply_min_p(l, min_p)
+    l = plain.apply_top_k(l, top_k)
+    return plain.apply_top_p(l, top_p)
+
+
+@pytest.mark.parametrize("V", [7, 1000, 20011])
+def test_filter_rows_against_the_plain_filters(V):
+    """Every filter alone, all together, a row left alone, ties at both thresholds."""
+    from spite_amd.sampling.sampler import Sampler, SamplingParams
+    g = torch.Generator().manual_seed(V)
+    cases = [dict(), dict(temperature=0.7), dict(top_k=3, temperature=1.0), dict(top_p=0.6, temperature=1.3),
+             dict(min_p=0.2, temperature=1.0), dict(penalty=1.4, last_n=0), dict(penalty=1.3, last_n=2, temperature=0.9),
+             dict(temperature=0.8, top_k=min(50, V - 1), top_p=0.9, min_p=0.01, penalty=1.2, last_n=0),
+             dict(top_k=4, temperature=1.0), dict(top_p=0.5, temperature=1.0),
+             dict(min_p=0.3, top_k=40, temperature=1.0), dict(top_k=5, temperature=1.0),
+             dict(top_p=0.999, temperature=1.0)]
+    n = len(cases)
+    logits = torch.randn(n, V, generator=g) * 3.0
+    # ties: rows 8 and 9 hold few distinct values, so that the k-th largest and the value at
+    # which the mass reaches p are shared by several elements (with a large vocabulary by more
+    # than the kernel sorts in one go: its digit-by-digit search runs)
+    few = 2 if V > 20000 else 4
+    logits[8] = torch.randint(0, few, (V,), generator=g).float()
+    logits[9] = torch.randint(0, few - 1 if few > 2 else 2, (V,), generator=g).float() * 0.5
+    # row 10: min-p leaves fewer values than top-k asks for.  Row 11: three values far above
+    # the rest, so that the fifth largest lies in the far tail.  Row 12: nearly all the mass.
+    logits[11, [1, V // 2, V - 1]] += 100.0
+    ctxs = [[int(x) for x in torch.randint(0, V, (9,), generator=g)] + [V + 5, -1] for _ in range(n)]
+    params = [SamplingParams(temperature=c.get("temperature", 0.0), top_k=c.get("top_k", 0), top_p=c.get("top_p", 1.0),
+                             min_p=c.get("min_p", 0.0), repetition_penalty=c.get("penalty", 1.0),
+                             repeat_last_n=c.get("last_n", 64)) for c in cases]
+    work = logits.to(DEV).clone()
+    Sampler(DEV)._filter(work, params, ctxs)
+    got = work.cpu()
+    for r, c in enumerate(cases):
+        if not params[r].filters():
+            assert torch.equal(got[r], logits[r]), r          # rows that ask for nothing are not touched
+            continue
+        want = _filter_case(logits[r], [t for t in ctxs[r]], **c)
+        assert torch.equal(torch.isinf(got[r]), torch.isinf(want)), (r, c, int(torch.isinf(got[r]).sum()), int(torch.isinf(want).sum()))
+        keep = ~torch.isinf(want)
+        assert torch.equal(got[r][keep], want[keep]), (r, c)
+    # top-k keeps every element equal to the k-th largest; top-p the first of the equal ones
+    kept8 = (~torch.isinf(got[8])).nonzero().flatten()
+    assert len(kept8) >= 4
+    if int((logits[8] == logits[8].max()).sum()) >= 4:
+        assert bool((logits[8][kept8] == logits[8].max()).all())
+    kept9 = (~torch.isinf(got[9])).nonzero().flatten().tolist()
+    top = (logits[9] == logits[9].max()).nonzero().flatten().tolist()
+    assert kept9 == top[:len(kept9)] or set(top) <= set(kept9)
