@@ -66,9 +66,16 @@ class StepMeta:
                     raise EngineError(f"entry {i}: wanted place {w} outside its {counts[i]} tokens")
                 rows.append(int(cu[i]) + int(w))
         n_out = len(rows)
+        # single decoded tokens that lead a mixed step (the scheduler's order): the mixer may give
+        # them to its decode kernel and only the portions behind them to the prefill kernel
+        lead = 0
+        while lead < n and counts[lead] == 1:
+            lead += 1
+        if lead == n:
+            lead = 0
         # layout of the one int32 buffer
         sizes = [("token_ids", T), ("positions", T), ("seq_of_token", T), ("cu_seqlens", n + 1),
-                 ("seq_slots", n), ("seq_starts", n), ("logit_rows", n_out)]
+                 ("seq_slots", n), ("seq_starts", n), ("logit_rows", n_out), ("cu_tail", n - lead + 1 if lead else 0)]
         for g in range(n_groups):
             sizes += [(f"slot_map{g}", T), (f"table{g}", n * widths[g])]
         offs, total = {}, 0
@@ -83,6 +90,8 @@ class StepMeta:
             hv["positions"][cu[i]:cu[i + 1]] = np.arange(starts[i], starts[i] + counts[i], dtype=np.int32)
             hv["seq_of_token"][cu[i]:cu[i + 1]] = i
         hv["cu_seqlens"][:] = cu
+        if lead:
+            hv["cu_tail"][:] = cu[lead:] - cu[lead]
         hv["seq_slots"][:] = slots
         hv["seq_starts"][:] = starts
         hv["logit_rows"][:] = np.asarray(rows, dtype=np.int32)
@@ -97,7 +106,8 @@ class StepMeta:
             cu_seqlens=dv["cu_seqlens"], seq_slots=dv["seq_slots"], seq_starts=dv["seq_starts"],
             logit_rows=dv["logit_rows"], n_out=n_out,
             host=HostBatch(slots=slots, starts=starts, counts=counts, cu_seqlens=cu),
-            decode_only=bool(n > 0 and counts.max() == 1), max_count=int(counts.max()) if n else 0)
+            decode_only=bool(n > 0 and counts.max() == 1), max_count=int(counts.max()) if n else 0,
+            lead_singles=lead, cu_tail=dv["cu_tail"] if lead else None)
         self.host_tokens = tok[:T].copy()
 
     def layer_cache(self, cache: PagedCache, call: LayerCall) -> LayerCache:

@@ -60,6 +60,23 @@ class Attention(Mixer):
     def cache_need(self):
         return CacheNeed(kv=KVNeed(self.G, self.hd, self.visibility, self.span))
 
+    def _decode(self, q, o, ctx, cache, T):
+        """The split-KV kernel over the step's first T tokens, each the only one of its request."""
+        H, G, hd = self.H, self.G, self.hd
+        # split the keys so that about five hundred workgroups run (measured: more splits only
+        # add partial results to combine), each wave with at least one block of keys; the
+        # bound on the keys is the block table's width, so the launch is the same for every
+        # step of that shape
+        longest = cache.block_table.shape[1] * cache.page_size
+        if self.visibility != "full":
+            longest = min(longest, self.span + 32)
+        blocks = -(-longest // 32)
+        n_splits = max(1, min(-(-512 // (T * G)), -(-blocks // 4), 256))
+        scratch = ctx.ws.take((hipops.attn_decode_workspace(T, H, hd, n_splits) // 4,), torch.float32)
+        hipops.attn_decode(q, cache.k_pages, cache.v_pages, o, scratch, ctx.positions, ctx.seq_of_token,
+                           cache.block_table, T, H, G, hd, cache.page_size, self.visibility, self.span,
+                           self.scale, n_splits)
+
     def forward(self, x, ctx, cache):
         T = x.shape[0]
         H, G, hd = self.H, self.G, self.hd
@@ -79,23 +96,21 @@ class Attention(Mixer):
                             write_kv=cache.write, kv_tiled=cache.tiled)
         o = ws.take((T, H * hd), x.dtype)
         # the MFMA kernels read pages in operand order (bfloat16, sizes in multiples of 32)
-        if ctx.decode_only and cache.tiled and hd in (64, 128) and H // G <= 16:
-            # split the keys so that about five hundred workgroups run (measured: more splits only
-            # add partial results to combine), each wave with at least one block of keys; the
-            # bound on the keys is the block table's width, so the launch is the same for every
-            # step of that shape
-            longest = cache.block_table.shape[1] * cache.page_size
-            if self.visibility != "full":
-                longest = min(longest, self.span + 32)
-            blocks = -(-longest // 32)
-            n_splits = max(1, min(-(-512 // (T * G)), -(-blocks // 4), 256))
-            scratch = ws.take((hipops.attn_decode_workspace(T, H, hd, n_splits) // 4,), torch.float32)
-            hipops.attn_decode(q, cache.k_pages, cache.v_pages, o, scratch, ctx.positions, ctx.seq_of_token,
-                               cache.block_table, T, H, G, hd, cache.page_size, self.visibility, self.span,
-                               self.scale, n_splits)
-        elif cache.tiled and hd in (64, 128):
-            hipops.attn_prefill(q, cache.k_pages, cache.v_pages, o, ctx.positions, ctx.cu_seqlens, ctx.host.counts,
-                                cache.block_table, H, G, hd, cache.page_size, self.visibility, self.span, self.scale)
+        mfma = cache.tiled and hd in (64, 128)
+        if ctx.decode_only and mfma and H // G <= 16:
+            self._decode(q, o, ctx, cache, T)
+        elif mfma:
+            lead = ctx.lead_singles if H // G <= 16 else 0
+            if lead:
+                # decoded tokens of other requests beside prompt portions: a query alone would
+                # fill a 256-column tile of the prefill kernel with five columns
+                self._decode(q, o, ctx, cache, lead)
+                hipops.attn_prefill(q[lead:], cache.k_pages, cache.v_pages, o[lead:], ctx.positions[lead:], ctx.cu_tail,
+                                    ctx.host.counts[lead:], cache.block_table[lead:], H, G, hd, cache.page_size,
+                                    self.visibility, self.span, self.scale)
+            else:
+                hipops.attn_prefill(q, cache.k_pages, cache.v_pages, o, ctx.positions, ctx.cu_seqlens, ctx.host.counts,
+                                    cache.block_table, H, G, hd, cache.page_size, self.visibility, self.span, self.scale)
         else:
             hipops.attn_generic(q, cache.k_pages, cache.v_pages, o, ctx.positions, ctx.seq_of_token,
                                 cache.block_table, T, H, G, hd, cache.page_size, self.visibility, self.span,

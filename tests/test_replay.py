@@ -143,6 +143,38 @@ def test_mixed_with_pages_used_again(case):
     check(case, (H.collect(steps, out, case.cfg["vocab_size"]), H.routing_hints(case.cfg, steps, routing)), "mixed")
 
 
+def test_decoded_tokens_lead_a_mixed_step(case, monkeypatch):
+    """The scheduler's own order: one decoded token of each running request first, portions of
+    prompts behind them.  Where the MFMA attention kernels run, the mixer gives the leading
+    tokens to the decode kernel and the portions to the prefill kernel."""
+    from spite_amd.csrc import hipops
+    ids = list(case.reqs)[-3:]
+    a, b, c = (case.reqs[i] for i in ids)
+    ka, kb = len(a) - 3, len(b) - 3
+    cut = [0, len(c) * 2 // 5, len(c) * 4 // 5, len(c)]
+    steps = [{"step": 0, "entries": [{"id": ids[0], "tokens": a[:ka], "want": list(range(ka))}], "end": []},
+             {"step": 1, "entries": [{"id": ids[1], "tokens": b[:kb], "want": list(range(kb))}], "end": []}]
+    for j in range(3):
+        steps.append({"step": 2 + j, "entries": [
+            {"id": ids[0], "tokens": [a[ka + j]], "want": [0]}, {"id": ids[1], "tokens": [b[kb + j]], "want": [0]},
+            {"id": ids[2], "tokens": c[cut[j]:cut[j + 1]], "want": list(range(cut[j + 1] - cut[j]))}],
+            "end": ids if j == 2 else []})
+    calls = []
+    real = hipops.attn_decode
+
+    def counted(q, k, v, out, ws, pos, seq, bt, T, *args, **kw):
+        calls.append((T, pos.numel()))
+        return real(q, k, v, out, ws, pos, seq, bt, T, *args, **kw)
+    monkeypatch.setattr(hipops, "attn_decode", counted)
+    reqs = {i: case.reqs[i] for i in ids}
+    ps = PAGE[case.name]
+    check(case, case.replay(steps, sum(-(-len(t) // ps) * ps for t in reqs.values())), "decodes first", reqs)
+    if case.dtype == "bfloat16" and case.cfg["head_dim"] in (64, 128):
+        assert calls and all(T == 2 and n > 2 for T, n in calls), calls[:4]
+    else:
+        assert not calls
+
+
 def test_schedules_agree_with_each_other(case):
     need = ["whole", "tail", "portions", "mixed"]
     if any(k not in case.results for k in need):
