@@ -208,11 +208,9 @@ extern "C" int spite_gemm_skinny(const void* X, int ldx, const void* W, long w_g
         else variant = offsets && !glu ? 3 : 9;
     }
     switch (variant) {
-        case 1: return launch_skinny<1, 1, 4, 8>(SP_ARGS);
         case 2: return launch_skinny<2, 2, 2, 8>(SP_ARGS);
         case 3: return launch_skinny<2, 4, 2, 4>(SP_ARGS);
         case 4: return launch_skinny<2, 1, 4, 8>(SP_ARGS);
-        case 5: return launch_skinny<1, 1, 4, 4>(SP_ARGS);
         case 6: return launch_skinny<1, 1, 2, 8>(SP_ARGS);
         case 7: return launch_skinny<4, 1, 2, 8>(SP_ARGS);
         case 8: return launch_skinny<2, 1, 2, 8>(SP_ARGS);

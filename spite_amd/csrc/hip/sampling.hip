@@ -168,6 +168,28 @@ __device__ void sort_falling(unsigned long long* list, int n) {
         }
 }
 
+// ---- where a row's elements lie below its maximum: bins of a quarter (the last one open), and,
+// inside a run of those bins that holds too many elements to sort, 127 finer bins.
+struct Bins {
+    int lo0, hi0;          // the quarter bins of the candidates
+    bool fine;             // whether the finer bins cut the candidates down further
+    int lo1, hi1;          // then: the finer bins of the candidates
+    float s1;              // finer bins per quarter bin of the run
+};
+__device__ __forceinline__ int bin_coarse(float mx, float x) { return (int)fminf((mx - x) * 4.0f, (float)(TP_BINS - 1)); }
+__device__ __forceinline__ int bin_fine(float mx, float x, int lo0, float s1) {
+    return (int)fminf(fmaxf(((mx - x) * 4.0f - (float)lo0) * s1, 0.f), (float)(TP_BINS - 2));
+}
+// 0: above the candidates (it stays for certain), 1: a candidate, 2: below them
+__device__ __forceinline__ int bin_class(const Bins& b, float mx, float x) {
+    const int c = bin_coarse(mx, x);
+    if (c < b.lo0) return 0;
+    if (c > b.hi0) return 2;
+    if (!b.fine) return 1;
+    const int f = bin_fine(mx, x, b.lo0, b.s1);
+    return f < b.lo1 ? 0 : (f > b.hi1 ? 2 : 1);
+}
+
 // The largest key t such that weight(keys >= t) reaches the goal, where an element weighs 1
 // (MASS = false: goal = k, the k-th largest key) or exp(l - mx) (MASS = true: goal = p as a
 // share of `total`).  `above` returns the weight of the keys greater than the result.
@@ -247,44 +269,57 @@ void filter_rows_kernel(float* __restrict__ work, int ld, int V, int n_rows, con
         each_of_mine(row, V, [&](int i, float x) { if (x < thresh) row[i] = -INFINITY; });
     }
     if (top_k > 0 && top_k < V) {
-        // counts by distance from the maximum, in bins of a quarter, name the bin of the k-th
-        // largest element; if it holds few, they are sorted in LDS
+        // counts by distance from the maximum name the bin of the k-th largest element (if that
+        // bin is crowded, finer bins inside it do); its elements are sorted in LDS
         int* hist_n = (int*)buckets;                                       // [TP_BINS]
         unsigned long long* list = (unsigned long long*)buckets + TP_BINS; // [TP_LIST]
         for (int j = tid; j < TP_BINS; j += FILT_NT) hist_n[j] = 0;
         if (tid == 0) cut = 0;
         __syncthreads();
-        auto bin_of = [&](float x) { return (int)fminf((mx - x) * 4.0f, (float)(TP_BINS - 1)); };
         each_of_mine(row, V, [&](int, float x) {
-            const int bin = bin_of(x);
+            const int bin = bin_coarse(mx, x);
             if (bin < TP_BINS - 1 || x > -INFINITY) atomicAdd(&hist_n[bin], 1);     // the open bin counts what is finite
         });
         __syncthreads();
-        int before = 0, bin_k = -1;
+        Bins b = {-1, -1, false, 0, 0, 0.f};
+        int before = 0;
         for (int j = 0; j < TP_BINS - 1; ++j) {
-            if (before + hist_n[j] >= top_k) { bin_k = j; break; }
+            if (before + hist_n[j] >= top_k) { b.lo0 = b.hi0 = j; break; }
             before += hist_n[j];
         }
-        float thresh;
-        if (bin_k < 0 && before + hist_n[TP_BINS - 1] < top_k) {
-            thresh = -INFINITY;                        // fewer than k finite values: all of them stay
+        const bool all_stay = b.lo0 < 0 && before + hist_n[TP_BINS - 1] < top_k;   // fewer than k finite values
+        int n_cand = b.lo0 >= 0 ? hist_n[b.lo0] : 0;
+        __syncthreads();
+        if (b.lo0 >= 0 && n_cand > TP_LIST) {
+            b.s1 = (float)(TP_BINS - 1);
+            for (int j = tid; j < TP_BINS; j += FILT_NT) hist_n[j] = 0;
             __syncthreads();
-        } else if (bin_k >= 0 && hist_n[bin_k] <= TP_LIST) {
-            const int n_cand = hist_n[bin_k];
+            each_of_mine(row, V, [&](int, float x) {
+                if (bin_coarse(mx, x) == b.lo0) atomicAdd(&hist_n[bin_fine(mx, x, b.lo0, b.s1)], 1);
+            });
+            __syncthreads();
+            for (int j = 0; j < TP_BINS - 1; ++j) {
+                if (before + hist_n[j] >= top_k) { b.fine = true; b.lo1 = b.hi1 = j; n_cand = hist_n[j]; break; }
+                before += hist_n[j];
+            }
+            __syncthreads();
+        }
+        float thresh;
+        if (all_stay) {
+            thresh = -INFINITY;
+        } else if (b.lo0 >= 0 && n_cand <= TP_LIST) {
             int n_pad = 64;
             while (n_pad < n_cand) n_pad <<= 1;
-            __syncthreads();
             for (int j = tid; j < n_pad; j += FILT_NT) list[j] = 0;
             __syncthreads();
             each_of_mine(row, V, [&](int, float x) {
-                if (bin_of(x) == bin_k) list[atomicAdd(&cut, 1)] = float_key(x);
+                if (bin_class(b, mx, x) == 1) list[atomicAdd(&cut, 1)] = float_key(x);
             });
             __syncthreads();
             sort_falling(list, n_pad);
             thresh = key_float((uint32_t)list[top_k - before - 1]);
             __syncthreads();
         } else {
-            __syncthreads();
             double above;
             thresh = key_float(select_key<false>(row, V, mx, 1.0, (double)top_k, above, sh, buckets));
         }
@@ -300,49 +335,75 @@ void filter_rows_kernel(float* __restrict__ work, int ld, int V, int n_rows, con
         // sums do not depend on the order of the atomic adds) and counts by distance from the
         // maximum, in bins of a quarter.  They tell in which bins the boundary can lie: the
         // elements above those bins stay for certain, the ones below go, and the elements of
-        // the bins themselves, if they are few, are sorted in LDS.
+        // the bins themselves are sorted in LDS; if they are too many for that, finer bins
+        // inside those bins cut them down first.
         unsigned long long* hist_m = (unsigned long long*)buckets;        // [TP_BINS]
         int* hist_n = (int*)(hist_m + TP_BINS);                            // [TP_BINS]
         unsigned long long* list = hist_m + 2 * TP_BINS;                   // [TP_LIST]
+        const double FIX = 1099511627776.0;                                // 2^40
         for (int j = tid; j < TP_BINS; j += FILT_NT) { hist_m[j] = 0; hist_n[j] = 0; }
         if (tid == 0) cut = 0;
         __syncthreads();
-        auto bin_of = [&](float x) { return (int)fminf((mx - x) * 4.0f, (float)(TP_BINS - 1)); };
         double part = 0.0;
         each_of_mine(row, V, [&](int, float x) {
             const float e = expf(x - mx);
             part += (double)e;
-            const int bin = bin_of(x);
+            const int bin = bin_coarse(mx, x);
             if (bin < TP_BINS - 1) {
-                atomicAdd(&hist_m[bin], (unsigned long long)((double)e * 1099511627776.0));   // 2^40
+                atomicAdd(&hist_m[bin], (unsigned long long)((double)e * FIX));
                 atomicAdd(&hist_n[bin], 1);
             }
         });
         const double total = block_sum1<double>(part, sh);
         // (block_sum1's barriers also order the atomics before the reads below)
-        int n_cand = 0, bin_lo = -1, bin_hi = -1;
-        {
-            // a bin's fixed-point mass is below the true one by less than its count
-            const double goal = top_p * total * 1099511627776.0;
-            double have = 0.0;
-            for (int j = 0; j < TP_BINS - 1; ++j) {
-                have += (double)hist_m[j];
-                if (bin_lo < 0 && have + (double)V >= goal * (1.0 - 1e-9)) bin_lo = j;
-                if (bin_lo >= 0) n_cand += hist_n[j];
-                if (have >= goal * (1.0 + 1e-9)) { bin_hi = j; break; }
-            }
+        // a bin's fixed-point mass is below the true one by less than its count: the first bin
+        // where the share may be reached, and the first where it is reached for certain
+        const double goal = top_p * total * FIX;
+        Bins b = {-1, -1, false, -1, -1, 0.f};
+        int n_cand = 0;
+        double have = 0.0, have_above = 0.0;           // fixed-point mass up to here / above the candidates
+        for (int j = 0; j < TP_BINS - 1; ++j) {
+            if (b.lo0 < 0 && have + (double)hist_m[j] + (double)V >= goal * (1.0 - 1e-9)) { b.lo0 = j; have_above = have; }
+            have += (double)hist_m[j];
+            if (b.lo0 >= 0) n_cand += hist_n[j];
+            if (have >= goal * (1.0 + 1e-9)) { b.hi0 = j; break; }
         }
-        if (bin_hi >= 0 && n_cand > 0 && n_cand <= TP_LIST) {
+        __syncthreads();
+        if (b.hi0 >= 0 && n_cand > TP_LIST) {
+            b.s1 = (float)(TP_BINS - 1) / (float)(b.hi0 - b.lo0 + 1);
+            for (int j = tid; j < TP_BINS; j += FILT_NT) { hist_m[j] = 0; hist_n[j] = 0; }
             __syncthreads();
+            each_of_mine(row, V, [&](int, float x) {
+                const int c = bin_coarse(mx, x);
+                if (c >= b.lo0 && c <= b.hi0) {
+                    const int f = bin_fine(mx, x, b.lo0, b.s1);
+                    atomicAdd(&hist_m[f], (unsigned long long)((double)expf(x - mx) * FIX));
+                    atomicAdd(&hist_n[f], 1);
+                }
+            });
+            __syncthreads();
+            have = have_above;
+            n_cand = 0;
+            for (int j = 0; j < TP_BINS - 1; ++j) {
+                if (b.lo1 < 0 && have + (double)hist_m[j] + (double)V >= goal * (1.0 - 1e-9)) b.lo1 = j;
+                have += (double)hist_m[j];
+                if (b.lo1 >= 0) n_cand += hist_n[j];
+                if (have >= goal * (1.0 + 1e-9)) { b.hi1 = j; break; }
+            }
+            b.fine = b.hi1 >= 0;
+            if (!b.fine) n_cand = TP_LIST + 1;         // (cannot happen: the run held the boundary) -> the search below
+            __syncthreads();
+        }
+        if (b.hi0 >= 0 && n_cand > 0 && n_cand <= TP_LIST) {
             int n_pad = 64;
             while (n_pad < n_cand) n_pad <<= 1;
             for (int j = tid; j < n_pad; j += FILT_NT) list[j] = 0;       // below every element
             __syncthreads();
-            double sure = 0.0;                                            // mass of the bins above
+            double sure = 0.0;                                            // mass of what lies above the candidates
             each_of_mine(row, V, [&](int i, float x) {
-                const int bin = bin_of(x);
-                if (bin < bin_lo) sure += (double)expf(x - mx);
-                else if (bin <= bin_hi) list[atomicAdd(&cut, 1)] = composite(x, i);
+                const int c = bin_class(b, mx, x);
+                if (c == 0) sure += (double)expf(x - mx);
+                else if (c == 1) list[atomicAdd(&cut, 1)] = composite(x, i);
             });
             sure = block_sum1<double>(sure, sh);
             sort_falling(list, n_pad);

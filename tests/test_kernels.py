@@ -185,7 +185,7 @@ def test_gemm_generic(M, N, K, dtype, out_dtype, glu, grouped):
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES + [(3, 40, 8), (12, 16, 4104)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("glu,grouped", [(False, False), (True, False), (False, True), (True, True)])
-@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10])
+@pytest.mark.parametrize("variant", [2, 3, 4, 6, 7, 8, 9, 10])
 def test_gemm_skinny(M, N, K, out_dtype, glu, grouped, variant):
     run_gemm(ops().gemm_skinny, torch.bfloat16, out_dtype, M, N, K, glu, grouped, variant=variant)
 
@@ -619,7 +619,8 @@ def test_filter_rows_against_the_plain_filters(V):
              dict(temperature=0.8, top_k=min(50, V - 1), top_p=0.9, min_p=0.01, penalty=1.2, last_n=0),
              dict(top_k=4, temperature=1.0), dict(top_p=0.5, temperature=1.0),
              dict(min_p=0.3, top_k=40, temperature=1.0), dict(top_k=5, temperature=1.0),
-             dict(top_p=0.999, temperature=1.0)]
+             dict(top_p=0.999, temperature=1.0), dict(top_p=0.9, temperature=1.0), dict(top_k=300, temperature=1.0),
+             dict(top_k=37, top_p=0.5, temperature=1.0)]
     n = len(cases)
     logits = torch.randn(n, V, generator=g) * 3.0
     # ties: rows 8 and 9 hold few distinct values, so that the k-th largest and the value at
@@ -631,6 +632,9 @@ def test_filter_rows_against_the_plain_filters(V):
     # row 10: min-p leaves fewer values than top-k asks for.  Row 11: three values far above
     # the rest, so that the fifth largest lies in the far tail.  Row 12: nearly all the mass.
     logits[11, [1, V // 2, V - 1]] += 100.0
+    # rows 13 to 15: nearly flat (what random weights give): one bin of the kernel's first look
+    # holds everything, its finer bins have to tell the elements apart
+    logits[13:16] *= 0.004
     ctxs = [[int(x) for x in torch.randint(0, V, (9,), generator=g)] + [V + 5, -1] for _ in range(n)]
     params = [SamplingParams(temperature=c.get("temperature", 0.0), top_k=c.get("top_k", 0), top_p=c.get("top_p", 1.0),
                              min_p=c.get("min_p", 0.0), repetition_penalty=c.get("penalty", 1.0),
