@@ -190,8 +190,7 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
             for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s[c][tt][i]);
-            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            mx = rows4_max(mx);
             const float m_new = fmaxf(m_run[c], mx * scale_log2e);
             // a column with nothing visible so far keeps m = -inf: its weights are zero, not NaN
             const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
@@ -205,8 +204,7 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
                     sum += e;
                     pf[c][tt >> 1][(tt & 1) * 4 + i] = (bf16)e;
                 }
-            sum += __shfl_xor(sum, 16, 64);
-            sum += __shfl_xor(sum, 32, 64);
+            sum = rows4_sum(sum);
             l_run[c] = l_run[c] * alpha[c] + sum;
             m_run[c] = m_new;
         }

@@ -97,6 +97,22 @@ __device__ __forceinline__ bool sp_find_tile(const int* offsets, int n_groups, i
     return false;
 }
 
+// Maximum / sum over the four lanes n, n+16, n+32, n+48 of a wave (the four rows of 16 lanes that
+// hold one MFMA column), the result in all four.  The row swaps are vector instructions: no
+// trip through the LDS crossbar as a shuffle across rows takes.
+__device__ __forceinline__ float rows4_max(float v) {
+    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float rows4_sum(float v) {
+    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 // Sum over a workgroup of NT threads (NT a multiple of 64, at most 1024); every thread
 // gets the result.  `red` is shared scratch of at least NT/64 floats; two barriers.
 template <int NT>
