@@ -277,7 +277,8 @@ class Engine:
         the caller has not done so; with ``commit`` the positions count as cached afterwards
         and pages that no later query can read are given back.  ``trace``, a dict, is a
         testing aid: parts leave what they decided in it (``moe_experts``: one int32 tensor
-        ``[tokens]`` per layer call with experts, in the order of the calls)."""
+        ``[tokens]`` per layer call with experts, in the order of the calls); a list under
+        ``take_experts`` gives them the experts to take instead of their routers' choice."""
         if not entries:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
         seen = set()

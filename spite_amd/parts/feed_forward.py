@@ -93,6 +93,17 @@ class MoeTop1Sigmoid(FeedForward):
         ws = ctx.ws
         expert = ws.take((T,), torch.int32)
         weight = ws.take((T,), torch.float32)
+        trace = ctx.extras.get("trace")
+        if trace is not None and trace.get("take_experts"):
+            # a testing aid: the experts are given (one tensor per call, in the order of the
+            # calls), each with the weight that its own logit gives; every other logit is
+            # taken out before the plan is made
+            take = trace["take_experts"].pop(0).to(device=x.device, dtype=torch.int64).view(T, 1)
+            logits = projected
+            if logits is None:
+                logits = ws.take((T, E), torch.float32)
+                hipops.gemm_generic(x32, self.w_router, logits, T, E, d)
+            projected = torch.full_like(logits, float("-inf")).scatter_(1, take, logits.gather(1, take))
         if projected is None:
             hipops.router_top1(x32, self.w_router, expert, weight)
         n = 2 * T if self.fused_shared else T
@@ -101,8 +112,8 @@ class MoeTop1Sigmoid(FeedForward):
         groups = E + 1 if self.fused_shared else E
         offsets = ws.take((groups + 1,), torch.int32)
         hipops.moe_plan(expert, weight, src, scale, dst, offsets, T, E, self.fused_shared, logits=projected)
-        if ctx.extras.get("trace") is not None:      # a testing aid: which expert each row took
-            ctx.extras["trace"].setdefault("moe_experts", []).append(expert.clone())
+        if trace is not None:                         # a testing aid: which expert each row took
+            trace.setdefault("moe_experts", []).append(expert.clone())
         act = ws.take((n, F), x.dtype)
         shape = grouped_tile_shape(T, E, groups - E) if T > SKINNY_MAX_ROWS else 0
         linear(x, self.w_gate_up, act, glu=True, offsets=offsets, n_groups=groups, a_rows=src, a_scale=scale, rows=n,

@@ -77,9 +77,10 @@ def random_tokens(vocab: int, n: int, seed: int):
 
 
 # ------------------------------------------------------------------ replay
-def run_trace_inprocess(engine, steps, routing=None):
+def run_trace_inprocess(engine, steps, routing=None, take=None):
     """Feeds ``steps`` (dicts of the trace format) to an Engine; returns {step: logits[wanted, V]}.
-    ``routing`` (a dict) receives {step: [experts of every token, one array per layer with experts]}."""
+    ``routing`` (a dict) receives {step: [experts of every token, one array per layer with experts]};
+    ``take`` (such a dict from another run) makes the engine take those experts."""
     from spite_amd.engine.engine import StepEntry
     slots, out = {}, {}
     for rec in steps:
@@ -88,7 +89,9 @@ def run_trace_inprocess(engine, steps, routing=None):
             if e["id"] not in slots:
                 slots[e["id"]] = engine.admit()
             entries.append(StepEntry(slots[e["id"]], e["tokens"], e.get("want", [])))
-        trace = {} if routing is not None else None
+        trace = {} if routing is not None or take is not None else None
+        if take is not None:
+            trace["take_experts"] = [torch.from_numpy(np.asarray(t)) for t in take[rec["step"]]]
         logits = engine.step(entries, trace=trace)
         if logits.shape[0]:
             out[rec["step"]] = logits.detach().cpu().numpy().copy()
