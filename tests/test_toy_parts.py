@@ -200,3 +200,81 @@ def test_the_same_toy_parts_in_bfloat16():
     # an expert chosen differently at a near tie of the router would show as an error of the
     # logits' own size; rounding to bfloat16 along two layers stays a few percent of it
     assert err < 0.06 * abs(ref).max(), (err, abs(ref).max())
+
+
+def test_a_toy_architecture_is_registered_by_name_and_served_from_a_folder(tmp_path):
+    """A whole architecture defined here: its config.json keys, its reader, its list of parts.
+    Registered under a name of its own, it goes through the framework's entry points unchanged:
+    the random-weights mode writes its folder, the engine picks the model class by config.json,
+    ``generate`` and the trace program run it."""
+    import json
+    import os
+    from dataclasses import dataclass
+    from spite_amd import Engine
+    from spite_amd.config.registry import register_architecture, registered_architectures
+    from spite_amd.parts.base import PartSpec, BlockSpec, LayerCall, ModelSpec
+    from spite_amd.weights.random_init import write_random_model
+    define_parts()
+
+    @dataclass
+    class ToyConfig:
+        width: int
+        depth: int
+        heads: int
+        words: int
+        window: int
+        ln_eps: float
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(**{k: raw[k] for k in ("width", "depth", "heads", "words", "window", "ln_eps")})
+
+    def build(cfg):
+        hd = cfg.width // cfg.heads
+        blocks = []
+        for L in range(cfg.depth):
+            p = f"toy.{L}."
+            ln = lambda n: PartSpec("toy_layernorm", {"width": cfg.width, "eps": cfg.ln_eps},
+                                    {"weight": p + n + ".w", "bias": p + n + ".b"})
+            mixer = PartSpec("attention", dict(hidden_size=cfg.width, n_heads=cfg.heads, n_kv_heads=1, head_dim=hd,
+                                               position=PartSpec("toy_scale", {"head_dim": hd}),
+                                               visibility="window", span=cfg.window, qk_norm=False, qk_norm_eps=1e-6,
+                                               temperature=None),
+                             dict({k: p + k for k in ("q_proj", "k_proj", "v_proj", "o_proj")}, **{"position.freq": p + "freq"}))
+            ffn = PartSpec("dense_glu", dict(hidden_size=cfg.width, intermediate_size=2 * cfg.width),
+                           {k: p + k for k in ("gate_proj", "up_proj", "down_proj")})
+            blocks.append(BlockSpec("prenorm", ln("ln1"), mixer, ln("ln2"), ffn))
+        # the second layer runs twice, each time over a cache of its own
+        order = [LayerCall(block=i, cache=i, write=True) for i in range(cfg.depth)] + [LayerCall(block=1, cache=cfg.depth, write=True)]
+        return ModelSpec(architecture="ToyWindowLM", vocab_size=cfg.words, hidden_size=cfg.width, blocks=blocks, order=order,
+                         final_norm=PartSpec("rms", {"width": cfg.width, "eps": 1e-5}, {"weight": "toy.out_norm"}),
+                         embed_name="toy.words", head_name=None, eos_token_ids=(), max_position=256)
+
+    register_architecture("ToyWindowLM", ToyConfig.from_dict, build)
+    assert "ToyWindowLM" in registered_architectures()
+    folder = str(tmp_path / "toy")
+    raw = dict(architectures=["ToyWindowLM"], width=48, depth=2, heads=3, words=77, window=5, ln_eps=1e-4,
+               torch_dtype="float32")
+    write_random_model(folder, raw, seed=5, std=0.2)
+    assert json.load(open(os.path.join(folder, "config.json")))["architectures"] == ["ToyWindowLM"]
+    eng = Engine(folder, dtype="float32", page_size=4, cache_tokens=128, max_requests=3)
+    assert eng.spec.architecture == "ToyWindowLM" and len(eng.spec.order) == 3
+    # the head is tied to the embedding; whole, token by token and mixed agree (no plain
+    # implementation of this model exists: the engine is held against itself)
+    reqs = {"x": H.random_tokens(77, 21, 1), "y": H.random_tokens(77, 10, 2)}
+    whole = H.collect(H.schedule_whole(reqs), H.run_trace_inprocess(eng, H.schedule_whole(reqs)), 77)
+    for steps in (H.schedule_tail_one_by_one(reqs, tail=6), H.schedule_mixed(reqs, seed=2, max_live=2)):
+        d, where = H.max_diff(H.collect(steps, H.run_trace_inprocess(eng, steps), 77), whole)
+        assert d < 1e-4, (d, where)
+    # the window: a token's logits depend on the last tokens only (two runs of windowed layers
+    # and one more reach back 3 * (window - 1) positions)
+    long = H.random_tokens(77, 40, 3)
+    other = H.random_tokens(77, 40, 4)[:20] + long[20:]
+    rows = {}
+    for name, toks in (("long", long), ("other", other)):
+        s = {name: toks}
+        rows[name] = H.collect(H.schedule_whole(s), H.run_trace_inprocess(eng, H.schedule_whole(s)), 77)
+    assert abs(rows["long"][("long", 39)] - rows["other"][("other", 39)]).max() < 1e-5
+    assert abs(rows["long"][("long", 24)] - rows["other"][("other", 24)]).max() > 1e-3
+    out = eng.generate([long[:7]], max_tokens=5)
+    assert len(out[0]) == 5 and all(0 <= t < 77 for t in out[0])
