@@ -123,6 +123,25 @@ def routing_hints(cfg, steps, routing):
     return hints
 
 
+def experts_to_take(cfg, steps, hints):
+    """{step: [experts of the step's tokens, one array per layer with experts]} from
+    {request: {layer: [expert at every position]}}: what ``routing_hints`` returns, cut the way
+    ``steps`` cuts the requests."""
+    layers = moe_layers(cfg)
+    fed, take = {}, {}
+    for rec in steps:
+        per_layer = [[] for _ in layers]
+        for e in rec["entries"]:
+            at, n = fed.get(e["id"], 0), len(e["tokens"])
+            for k, L in enumerate(layers):
+                per_layer[k].extend(hints[e["id"]][L][at:at + n])
+            fed[e["id"]] = at + n
+        take[rec["step"]] = [np.asarray(x, dtype=np.int32) for x in per_layer]
+        for rid in rec.get("end", []):
+            fed.pop(rid, None)
+    return take
+
+
 def run_trace_program(model_dir, dtype, steps, max_tokens, extra=(), routing=None):
     """The same through ``bin/trace_run`` as a child process, one step at a time."""
     out_dir = tempfile.mkdtemp(prefix="trace_out_")
