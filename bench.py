@@ -89,6 +89,36 @@ def prefill_flops(cfg, L, T, past=0):
     return L * 2 * proj * T + 4 * pairs * H * hd + 2 * T * (n_moe * moe + (L - n_moe) * dense) + 2 * d * V
 
 
+def sampling_only(V, rows, steps):
+    """Times the sampler alone (no model): rows of random logits, peaked like a trained model's or
+    flat like a random one's, through the option sets that the command line offers."""
+    import numpy as np
+    import torch
+    from spite_amd.sampling.sampler import Sampler, SamplingParams
+    dev = torch.device("cuda:0")
+    sampler = Sampler(dev)
+    g = torch.Generator(device=dev).manual_seed(0)
+    out = {}
+    for spread, scale in (("peaked", 3.0), ("flat", 0.05)):
+        logits = torch.randn(rows, V, device=dev, generator=g) * scale
+        for name, p in (("greedy", SamplingParams()), ("temperature", SamplingParams(temperature=0.8)),
+                        ("top_p", SamplingParams(temperature=0.8, top_p=0.95)),
+                        ("top_k", SamplingParams(temperature=0.8, top_k=40)),
+                        ("all", SamplingParams(temperature=0.8, top_k=40, top_p=0.95, min_p=0.05, repetition_penalty=1.1))):
+            params, ctx, st = [p] * rows, [[1, 2, 3]] * rows, [1] * rows
+            for _ in range(2):
+                sampler.sample(logits, params, ctx, st)
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            for _ in range(steps):
+                sampler.sample(logits, params, ctx, st)
+            torch.cuda.synchronize()
+            out[f"{spread}_{name}_ms"] = round((time.perf_counter() - t) / steps * 1e3, 3)
+            log(f"sampling {rows} rows of {V}, {spread} logits, {name}: {out[f'{spread}_{name}_ms']} ms a call")
+    print(json.dumps({"metric": "sampling only", "value": None, "n_gpus": 1, "rows": rows, "vocab": V, "ms_per_call": out}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -107,7 +137,7 @@ def main() -> int:
     ap.add_argument("--moe-step", type=int, default=None,
                     help="every how many layers the feed-forward is the experts' (default 1; 2 = dense layers between)")
     ap.add_argument("--no-graphs", action="store_true", help="run decode steps eagerly (for kernel traces)")
-    ap.add_argument("--phase", default="all", choices=["all", "decode", "prefill"],
+    ap.add_argument("--phase", default="all", choices=["all", "decode", "prefill", "sampling"],
                     help="time only one phase (for kernel traces); the other's figures are null")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -120,6 +150,8 @@ def main() -> int:
     from spite_amd.sampling.sampler import Sampler, SamplingParams
 
     base = TINY if args.tiny else SCOUT
+    if args.phase == "sampling":
+        return sampling_only(base["vocab_size"], args.batch, args.steps)
     layers_full = base["num_hidden_layers"]
     L = args.layers or layers_full
     cfg = dict(base, num_hidden_layers=L, no_rope_layers=None)

@@ -1,8 +1,7 @@
 // Token choice from fp32 logits rows: arg-max (the lowest index wins a tie) and the
 // inverse-CDF draw of crates/spite-sampling/src/lib.rs:247-265 (m = max, total = sum
 // exp(l-m), the first index whose running sum reaches u*total, arg-max if rounding leaves
-// none).  One workgroup per row; each thread owns one contiguous slice of the row, so the
-// running sum walks the row in index order.
+// none).  One workgroup per row.
 #include "common.h"
 #include <type_traits>
 
@@ -28,50 +27,86 @@ __device__ void block_argmax(float& v, int& i, float* sv, int* si) {
     __syncthreads();
 }
 
+// The draw: masses exp(l/T - max) are summed over spans of SAMP_SPAN consecutive elements, a
+// span by one wave (sixteen loads of 64 neighbouring elements, one sum across the lanes), the
+// spans in index order; the first span, then the first run of 64 in it, then the first element
+// at which the running sum reaches u * total is the answer.
+#define SAMP_SPAN 1024
 __global__ __launch_bounds__(SAMP_NT)
 void sample_rows_kernel(const float* __restrict__ logits, int ld, int V, const float* __restrict__ temperature,
                         const float* __restrict__ uniform, int* __restrict__ out) {
     __shared__ float sv[SAMP_NT / 64];
     __shared__ int si[SAMP_NT / 64];
-    __shared__ float part[SAMP_NT];
-    __shared__ int found;
-    const int r = blockIdx.x, tid = threadIdx.x;
+    __shared__ int at_span;
+    __shared__ float before, goal;
+    extern __shared__ float span_sum[];             // [spans]
+    const int r = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const float* row = logits + (size_t)r * ld;
     const float temp = temperature ? temperature[r] : 0.f;
-    const int per = (V + SAMP_NT - 1) / SAMP_NT;
-    const int b = tid * per, e = (b + per < V) ? b + per : V;
 
     // arg-max: neighbouring threads read neighbouring elements; a thread meets its indices in
     // rising order, so "greater than" keeps the lowest index of equal values
     float bv = 0.f; int bi = -1;
-    for (int i = tid; i < V; i += SAMP_NT) {
-        const float x = row[i];
-        if (bi < 0 || x > bv) { bv = x; bi = i; }
+    for (int base = tid; base < V; base += 16 * SAMP_NT) {       // sixteen loads in flight
+        float x[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const int i = base + u * SAMP_NT;
+            x[u] = i < V ? row[i] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const int i = base + u * SAMP_NT;
+            if (i < V && (bi < 0 || x[u] > bv)) { bv = x[u]; bi = i; }
+        }
     }
     block_argmax(bv, bi, sv, si);
     if (temp <= 0.f) { if (tid == 0) out[r] = bi; return; }
 
-    // masses relative to the maximum of l/temperature
     const float mx = bv / temp;
-    float s = 0.f;
-    for (int i = b; i < e; ++i) s += expf(row[i] / temp - mx);
-    part[tid] = s;
-    if (tid == 0) found = 0x7fffffff;
-    __syncthreads();
-    float excl = 0.f, total = 0.f;
-    for (int k = 0; k < SAMP_NT; ++k) { if (k == tid) excl = total; total += part[k]; }
-    const float target = uniform[r] * total;
-    // Every slice that starts below the target walks on from the sum of the slices before
-    // it; the lowest index that reaches the target is the answer.
-    if (b < e && (tid == 0 || excl < target)) {
-        float cum = excl;
-        for (int i = b; i < e; ++i) {
-            cum += expf(row[i] / temp - mx);
-            if (cum >= target) { atomicMin(&found, i); break; }
+    const int n_spans = (V + SAMP_SPAN - 1) / SAMP_SPAN;
+    for (int sp = wave; sp < n_spans; sp += SAMP_NT / 64) {
+        float x[SAMP_SPAN / 64];
+#pragma unroll
+        for (int u = 0; u < SAMP_SPAN / 64; ++u) {
+            const int i = sp * SAMP_SPAN + u * 64 + lane;
+            x[u] = i < V ? row[i] : -INFINITY;
         }
+        float s = 0.f;
+#pragma unroll
+        for (int u = 0; u < SAMP_SPAN / 64; ++u) s += expf(x[u] / temp - mx);      // (exp(-inf) = 0 past the end)
+        s = wave_sum(s);
+        if (lane == 0) span_sum[sp] = s;
     }
     __syncthreads();
-    if (tid == 0) out[r] = found != 0x7fffffff ? found : bi;
+    if (tid == 0) {
+        float total = 0.f;
+        for (int sp = 0; sp < n_spans; ++sp) total += span_sum[sp];
+        const float target = uniform[r] * total;
+        float cum = 0.f;
+        int sp = 0;
+        while (sp < n_spans - 1 && cum + span_sum[sp] < target) cum += span_sum[sp++];
+        at_span = sp; before = cum; goal = target;
+    }
+    __syncthreads();
+    if (wave == 0) {
+        // inside the span: run by run, the running sum over a run's lanes in index order
+        float cum = before;
+        int found = -1;
+        for (int u = 0; u < SAMP_SPAN / 64 && found < 0; ++u) {
+            const int i = at_span * SAMP_SPAN + u * 64 + lane;
+            float c = i < V ? expf(row[i] / temp - mx) : 0.f;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const float v = __shfl_up(c, o, 64);
+                if (lane >= o) c += v;
+            }
+            const unsigned long long hit = __ballot(i < V && cum + c >= goal);
+            if (hit) found = at_span * SAMP_SPAN + u * 64 + (__ffsll((long long)hit) - 1);
+            cum += __shfl(c, 63, 64);
+        }
+        if (lane == 0) out[r] = found >= 0 ? found : bi;
+    }
 }
 
 // ------------------------------------------------------------------ filters before the draw
@@ -83,8 +118,8 @@ void sample_rows_kernel(const float* __restrict__ logits, int ld, int V, const f
 // one; :147-180).  Dropped logits become -inf.  One workgroup per row; nothing is sorted:
 // the k-th largest value and the value at which the mass reaches p are found digit by digit
 // (four bits a pass) over an order-preserving integer image of the floats, with counts, or
-// masses in 64-bit floating point, per digit.  Every thread owns the elements tid, tid + NT,
-// ... of the row in all passes, and all sums run in a fixed order.
+// masses in 64-bit floating point, per digit.  Every thread owns the same elements of the row
+// in all passes, and all sums run in a fixed order.
 // `params` is [6][n_rows] doubles: on (0 = leave the row alone), temperature, ln(min_p)
 // (-inf = off), top_k (0 = off), top_p (>= 1 = off), penalty.
 #define FILT_NT 1024
@@ -99,8 +134,9 @@ __device__ __forceinline__ float key_float(uint32_t k) {
     return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
 }
 
-// f(i, row[i]) for the thread's elements tid, tid + NT, ...: sixteen loads are in flight at a time
-// (a pass is bound by the latency of its loads otherwise).
+// f(i, row[i]) for the thread's elements tid, tid + NT, ..., the same ones in every pass over a
+// row; sixteen loads are in flight at a time.  (16-byte loads of four neighbours were measured
+// slower: the passes are bound by their arithmetic and LDS traffic on the one CU, not by loads.)
 template <typename F>
 __device__ __forceinline__ void each_of_mine(const float* row, int V, F f) {
     constexpr int U = 16;
@@ -559,7 +595,9 @@ extern "C" int spite_sample_rows(const float* logits, int ld, int n_rows, int V,
     SP_REQUIRE(n_rows >= 0 && V > 0 && ld >= V, "sample: bad sizes rows=%d V=%d ld=%d", n_rows, V, ld);
     SP_REQUIRE(!temperature || uniform, "sample: temperatures without uniform draws");
     if (n_rows == 0) return 0;
-    sample_rows_kernel<<<n_rows, SAMP_NT, 0, st>>>(logits, ld, V, temperature, uniform, out);
+    const size_t lds = (size_t)((V + SAMP_SPAN - 1) / SAMP_SPAN) * sizeof(float);
+    SP_REQUIRE(lds <= 40 * 1024, "sample: a vocabulary of %d is beyond this kernel (at most %d)", V, 10 * 1024 * SAMP_SPAN);
+    sample_rows_kernel<<<n_rows, SAMP_NT, lds, st>>>(logits, ld, V, temperature, uniform, out);
     SP_LAUNCH_CHECK("sample_rows");
     return 0;
 }
