@@ -659,3 +659,42 @@ extern "C" int spite_convert(const void* in, int in_dtype, void* out, int out_dt
     SP_LAUNCH_CHECK("convert");
     return 0;
 }
+
+// ------------------------------------------------------------------ random weights
+// out[i] = mean + std * z(seed, key, i), z standard normal: element i of a tensor depends on the
+// seed, the tensor's key (a hash of its name) and i alone, not on the order in which tensors
+// or elements are drawn.  A 64-bit mix of (seed, key, i / 2) gives two uniform numbers, and
+// Box-Muller turns them into the normals of the elements i and i + 1.
+__device__ __forceinline__ unsigned long long mix64(unsigned long long x) {
+    x ^= x >> 30; x *= 0xbf58476d1ce4e5b9ull;
+    x ^= x >> 27; x *= 0x94d049bb133111ebull;
+    return x ^ (x >> 31);
+}
+template <typename T>
+__global__ __launch_bounds__(256)
+void randn_fill_kernel(T* __restrict__ out, size_t n, unsigned long long seed, unsigned long long key, float mean, float std) {
+    const unsigned long long base = mix64(seed * 0x9e3779b97f4a7c15ull + key);
+    const size_t pairs = (n + 1) / 2;
+    for (size_t j = (size_t)blockIdx.x * blockDim.x + threadIdx.x; j < pairs; j += (size_t)gridDim.x * blockDim.x) {
+        const unsigned long long h = mix64(base + j * 0xd1342543de82ef95ull);
+        const float u1 = ((float)(unsigned)(h >> 40) + 1.0f) * (1.0f / 16777216.0f);          // (0, 1]
+        const float u2 = (float)(unsigned)((h >> 16) & 0xffffff) * (1.0f / 16777216.0f);      // [0, 1)
+        const float r = sqrtf(-2.0f * logf(u1));
+        float sn, cs;
+        sincosf(6.283185307179586f * u2, &sn, &cs);
+        out[2 * j] = from_f32<T>(mean + std * r * cs);
+        if (2 * j + 1 < n) out[2 * j + 1] = from_f32<T>(mean + std * r * sn);
+    }
+}
+extern "C" int spite_randn_fill(void* out, int dtype, size_t n, unsigned long long seed, unsigned long long key,
+                                float mean, float std, hipStream_t st) {
+    SP_REQUIRE(std >= 0.f, "randn_fill: a deviation of %g", std);
+    if (n == 0) return 0;
+    const size_t blocks = ((n + 1) / 2 + 255) / 256;
+    const int grid = (int)(blocks < 16384 ? blocks : 16384);
+    if (dtype == SP_BF16) randn_fill_kernel<bf16><<<grid, 256, 0, st>>>((bf16*)out, n, seed, key, mean, std);
+    else if (dtype == SP_F32) randn_fill_kernel<float><<<grid, 256, 0, st>>>((float*)out, n, seed, key, mean, std);
+    else return sp_fail("randn_fill: unknown dtype %d", dtype);
+    SP_LAUNCH_CHECK("randn_fill");
+    return 0;
+}

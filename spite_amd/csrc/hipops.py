@@ -39,6 +39,7 @@ def lib():
             "spite_router_top1": [P, P, P, P, P, I, I, I, P],
             "spite_moe_plan": [P, P, P, P, P, P, P, I, I, I, P],
             "spite_convert": [P, I, P, I, c_size_t, P],
+            "spite_randn_fill": [P, I, c_size_t, ctypes.c_ulonglong, ctypes.c_ulonglong, F, F, P],
             "spite_gemm_generic": [P, I, P, L, I, P, I, I, I, I, I, P, I, P, P, P, I, P],
             "spite_attn_generic": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, I, P],
             "spite_sample_rows": [P, I, I, I, P, P, P, P],
@@ -201,6 +202,15 @@ def convert(src, dst):
         raise KernelError("convert: sizes differ")
     _check(lib().spite_convert(_ptr(src, "src"), dtype_code(src.dtype), _ptr(dst, "dst"), dtype_code(dst.dtype),
                                src.numel(), _stream()), "convert")
+
+
+def randn_fill(t, seed: int, key: int, mean: float = 0.0, std: float = 1.0):
+    """t[i] = mean + std * z(seed, key, i) with z standard normal: counter-based, so a tensor's
+    numbers depend on the seed, its key and the element's index alone."""
+    if not t.is_contiguous():
+        raise KernelError("randn_fill: the tensor must be contiguous")
+    _check(lib().spite_randn_fill(_ptr(t, "t"), dtype_code(t.dtype), t.numel(), int(seed) & ((1 << 64) - 1),
+                                  int(key) & ((1 << 64) - 1), float(mean), float(std), _stream()), "randn_fill")
 
 
 def gemm_generic(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None,

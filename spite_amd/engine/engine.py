@@ -203,9 +203,10 @@ class Engine:
         self.model.finish_loading()
 
     def _init_random(self, seed: int, std: float):
-        """Draws every tensor on the GPU in its resident dtype: N(0,std), norm weights 1+N(0,std)."""
-        gen = torch.Generator(device=self.device)
-        gen.manual_seed(int(seed))
+        """Draws every tensor on the GPU in its resident dtype: N(0,std), norm weights 1+N(0,std).
+        The numbers of a tensor depend on the seed, the tensor's name and the element's index
+        alone (``hipops.randn_fill``)."""
+        import zlib
         by_owner = {}
         for f, ps, owner, local in self.model.tensor_plan():
             if ps.kind == "int":
@@ -216,9 +217,7 @@ class Engine:
                 if ps.init == "zeros":
                     t.zero_()
                 else:
-                    t.normal_(0.0, std, generator=gen)
-                    if ps.init == "ones":
-                        t += 1.0
+                    hipops.randn_fill(t, seed, zlib.crc32(f.encode()), 1.0 if ps.init == "ones" else 0.0, std)
             by_owner.setdefault(id(owner), (owner, {}))[1][local] = t
         for owner, ts in by_owner.values():
             owner.load(ts)

@@ -658,3 +658,31 @@ def test_filter_rows_against_the_plain_filters(V):
     kept9 = (~torch.isinf(got[9])).nonzero().flatten().tolist()
     top = (logits[9] == logits[9].max()).nonzero().flatten().tolist()
     assert kept9 == top[:len(kept9)] or set(top) <= set(kept9)
+
+
+def test_randn_fill_is_normal_and_depends_on_seed_key_and_index_alone():
+    n = 1 << 20
+    a = torch.empty(n, device=DEV)
+    ops().randn_fill(a, 7, 99, 0.0, 1.0)
+    assert abs(float(a.mean())) < 5e-3 and abs(float(a.std()) - 1.0) < 5e-3
+    z = a.double().cpu()
+    # the shape of the distribution: its fourth moment, and the share beyond two deviations
+    assert abs(float((z ** 4).mean()) - 3.0) < 0.1 and abs(float((z.abs() > 2).double().mean()) - 0.0455) < 2e-3
+    # neighbours (the two normals of one pair, and those of adjacent pairs) are uncorrelated
+    for lag in (1, 2, 3):
+        assert abs(float((z[:-lag] * z[lag:]).mean())) < 5e-3
+    # the same call gives the same numbers; a longer tensor starts with them; mean and deviation scale them
+    b = torch.empty(n + 5, device=DEV)
+    ops().randn_fill(b, 7, 99, 1.0, 0.02)
+    assert torch.allclose(b[:n], 1.0 + 0.02 * a, atol=1e-6)
+    c = torch.empty(n, device=DEV)
+    ops().randn_fill(c, 7, 99, 0.0, 1.0)
+    assert torch.equal(a, c)
+    # another key or another seed: other numbers
+    for seed, key in ((7, 100), (8, 99)):
+        ops().randn_fill(c, seed, key, 0.0, 1.0)
+        assert abs(float((a * c).mean())) < 5e-3 and not torch.equal(a, c)
+    # bfloat16 holds the rounded values; an odd length fills its last element
+    h = torch.empty(1001, dtype=torch.bfloat16, device=DEV)
+    ops().randn_fill(h, 7, 99, 0.0, 1.0)
+    assert torch.equal(h, a[:1001].to(torch.bfloat16))
