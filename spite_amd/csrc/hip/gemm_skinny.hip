@@ -205,7 +205,10 @@ extern "C" int spite_gemm_skinny(const void* X, int ldx, const void* W, long w_g
             else variant = 8;
         }
         else if (max_rows <= 32) variant = !offsets && (size_t)N * K >= ((size_t)1 << 28) ? 10 : 2;
-        else variant = offsets && !glu ? 3 : 9;
+        // (groups of experts at 33 to 64 tokens hold a few rows each, only the shared one all:
+        // 32 columns a workgroup and a second row tile for that group beat 64 columns for all)
+        else if (offsets) variant = glu ? 2 : 10;
+        else variant = 9;
     }
     switch (variant) {
         case 2: return launch_skinny<2, 2, 2, 8>(SP_ARGS);
