@@ -31,7 +31,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restrict__ W, long w_group_stride,
                        TY* __restrict__ Y, int ldy, int M, int N, int K,
                        const int* __restrict__ offsets, int n_groups, const int* __restrict__ a_rows,
-                       const float* __restrict__ a_scale, const int* __restrict__ y_rows, int m_tiles, int n_tiles) {
+                       const float* __restrict__ a_scale, const int* __restrict__ y_rows, int m_tiles, int n_tiles,
+                       int k_splits, size_t split_stride) {
     static_assert(WN * WM == 8, "eight waves");
     constexpr int WS = 16 * NB;                     // slots of a wave: NB slot tiles
     constexpr int BM = WS * WM, BN = 64 * WN;
@@ -40,9 +41,13 @@ void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restri
 
     // Which tile.  Workgroups go to the eight XCDs in turn, each with an L2 of its own: XCD x
     // takes the x-th eighth of the tiles, ordered with the row tile running fastest.
-    const int per_xcd = (m_tiles * n_tiles + 7) / 8;
-    const int tile_id = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-    if (tile_id >= m_tiles * n_tiles) return;
+    // With k_splits > 1 a tile's sum over k is cut into that many runs, each a workgroup of its
+    // own that writes its partial sums to Y + run * split_stride (the caller adds them up).
+    const int units = m_tiles * n_tiles * k_splits;
+    const int per_xcd = (units + 7) / 8;
+    const int unit_id = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (unit_id >= units) return;
+    const int ks = unit_id % k_splits, tile_id = unit_id / k_splits;
     const int tile_m = tile_id % m_tiles, tile_n = tile_id / m_tiles;
     int g = 0, row0, row_end = M;
     if (offsets) {
@@ -72,7 +77,7 @@ void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restri
     // ---- W: the wave's four row bands
     //      plain: rows n0 + wn*64 + a*16; GLU: bands 0, 1 gate rows n0 + wn*32 + ..., bands 2, 3 the up rows N + ...
     constexpr int TG = GLU ? 2 : 4;          // bands that name distinct output columns
-    const int kt = K / 32;                   // tiles in a band
+    const int kt_all = K / 32;               // tiles in a band
     const bf16* wsrc[4];
     int ncol[4];                             // output column of the band's first row
 #pragma unroll
@@ -82,9 +87,17 @@ void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restri
         band = band < N / 16 ? band : N / 16 - 1;        // bands past N read the last band again
         if (GLU && a >= TG) band += N / 16;
         ncol[a] = n;
-        wsrc[a] = Wg + (size_t)band * kt * 512 + lane * 8;
+        wsrc[a] = Wg + (size_t)band * kt_all * 512 + lane * 8;
     }
-    const int nu = K / 64;
+    // this workgroup's run of 64-k steps
+    const int nu_all = K / 64, per_run = (nu_all + k_splits - 1) / k_splits;
+    const int u_first = ks * per_run;
+    const int nu = (u_first + per_run < nu_all ? u_first + per_run : nu_all) - u_first;     // > 0 by the caller's choice of k_splits
+#pragma unroll
+    for (int i = 0; i < XL; ++i) xsrc[i] += (size_t)u_first * 64;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) wsrc[a] += (size_t)u_first * 2 * 512;
+    Y += (size_t)ks * split_stride;
     auto load_x = [&](bf16x8 (&xr)[XL], int u) {
         const int k0 = (u < nu ? u : nu - 1) * 64;
 #pragma unroll
@@ -97,6 +110,7 @@ void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restri
             if (64 * (i + 1) <= BM || lrow + 64 * i < BM)
                 *(bf16x8*)(Xs + buf * (BM * TLD) + (lrow + 64 * i) * TLD + lchunk * 8) = xr[i];
     };
+    const int kt = 2 * nu;                   // 32-k tiles of the run
     auto load_w = [&](bf16x8 (&ws)[4], int t) {
         const size_t at = (size_t)(t < kt ? t : kt - 1) * 512;
 #pragma unroll
@@ -217,12 +231,12 @@ void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restri
 template <int WN, int WM, int NB, bool GLU, typename TY>
 static int launch_tiled_kernel(const void* X, int ldx, const void* W, long w_group_stride, void* Y, int ldy, int M, int N,
                                int K, const int* offsets, int n_groups, const int* a_rows, const float* a_scale,
-                               const int* y_rows, hipStream_t st) {
+                               const int* y_rows, int k_splits, size_t split_stride, hipStream_t st) {
     constexpr int BM = 16 * NB * WM, BN = 64 * WN;
     const int m_tiles = (M + BM - 1) / BM + (offsets ? n_groups : 0);
     const int ncols = GLU ? BN / 2 : BN;
     const int n_tiles = (N + ncols - 1) / ncols;
-    SP_REQUIRE((long)m_tiles * n_tiles < (1L << 30), "gemm_tiled: too many tiles");
+    SP_REQUIRE((long)m_tiles * n_tiles * k_splits < (1L << 30), "gemm_tiled: too many tiles");
     const size_t sh = (size_t)2 * BM * TLD * sizeof(bf16);
     static bool allowed = false;        // one flag per instantiation; more LDS than the default limit for WM = 2
     if (!allowed) {
@@ -231,9 +245,9 @@ static int launch_tiled_kernel(const void* X, int ldx, const void* W, long w_gro
         SP_REQUIRE(e == hipSuccess, "gemm_tiled: %zu bytes of LDS refused: %s", sh, hipGetErrorString(e));
         allowed = true;
     }
-    gemm_tiled_kernel<WN, WM, NB, GLU, TY><<<dim3((m_tiles * n_tiles + 7) / 8 * 8), 512, sh, st>>>(
+    gemm_tiled_kernel<WN, WM, NB, GLU, TY><<<dim3((m_tiles * n_tiles * k_splits + 7) / 8 * 8), 512, sh, st>>>(
         (const bf16*)X, ldx, (const bf16*)W, w_group_stride, (TY*)Y, ldy, M, N, K, offsets, n_groups, a_rows, a_scale,
-        y_rows, m_tiles, n_tiles);
+        y_rows, m_tiles, n_tiles, k_splits, split_stride);
     SP_LAUNCH_CHECK("gemm_tiled");
     return 0;
 }
@@ -243,10 +257,45 @@ static int launch_tiled(const void* X, int ldx, const void* W, long w_group_stri
                         int N, int K, const int* offsets, int n_groups, const int* a_rows, const float* a_scale,
                         const int* y_rows, int glu, hipStream_t st) {
 #define SP_TL(GLUV, TY) launch_tiled_kernel<WN, WM, NB, GLUV, TY>(X, ldx, W, w_group_stride, Y, ldy, M, N, K, offsets, n_groups, \
-                                                              a_rows, a_scale, y_rows, st)
+                                                              a_rows, a_scale, y_rows, 1, 0, st)
     if (glu) return y_dtype == SP_BF16 ? SP_TL(true, bf16) : SP_TL(true, float);
     return y_dtype == SP_BF16 ? SP_TL(false, bf16) : SP_TL(false, float);
 #undef SP_TL
+}
+
+// Sum of the partial products of a split call: out[m][n] = sum over runs of part[run][m][n].
+template <typename TY>
+__global__ void add_runs_kernel(const float* __restrict__ part, int runs, size_t stride, TY* __restrict__ out, int ldy, int M, int N) {
+    const size_t total = (size_t)M * N;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        float v = 0.f;
+        for (int r = 0; r < runs; ++r) v += part[(size_t)r * stride + i];
+        out[(i / N) * ldy + i % N] = from_f32<TY>(v);
+    }
+}
+
+// A plain product (no groups, no row lists, no GLU) over few tiles, the sum over k cut into
+// `k_splits` runs so that the chip is filled: `workspace` holds k_splits * M * N floats.
+extern "C" int spite_gemm_tiled_split(const void* X, int ldx, const void* W, void* Y, int y_dtype, int ldy, int M, int N,
+                                      int K, int k_splits, void* workspace, hipStream_t st) {
+    SP_REQUIRE(M > 0 && N > 0 && K > 0 && ldx >= K && ldy >= N, "gemm_tiled: bad sizes M=%d N=%d K=%d", M, N, K);
+    SP_REQUIRE(K % 64 == 0 && N % 16 == 0, "gemm_tiled: operand order needs K=%d a multiple of 64 and N=%d of 16", K, N);
+    SP_REQUIRE(ldx % 8 == 0, "gemm_tiled: the row stride %d must be a multiple of 8", ldx);
+    SP_REQUIRE(((uintptr_t)X & 15) == 0 && ((uintptr_t)W & 15) == 0, "gemm_tiled: operands must be 16-byte aligned");
+    SP_REQUIRE(y_dtype == SP_BF16 || y_dtype == SP_F32, "gemm_tiled: output dtype %d", y_dtype);
+    const int nu = K / 64;
+    SP_REQUIRE(k_splits >= 2 && workspace, "gemm_tiled: a split call needs at least two runs and a workspace");
+    SP_REQUIRE(((nu + k_splits - 1) / k_splits) * (k_splits - 1) < nu, "gemm_tiled: %d runs over %d steps leave a run empty", k_splits, nu);
+    const size_t stride = (size_t)M * N;
+    int rc = launch_tiled_kernel<8, 1, 8, false, float>(X, ldx, W, 0, workspace, N, M, N, K, nullptr, 1, nullptr, nullptr, nullptr,
+                                                        k_splits, stride, st);
+    if (rc) return rc;
+    const size_t blocks = (stride + 255) / 256;
+    const int grid = (int)(blocks < 8192 ? blocks : 8192);
+    if (y_dtype == SP_BF16) add_runs_kernel<bf16><<<grid, 256, 0, st>>>((const float*)workspace, k_splits, stride, (bf16*)Y, ldy, M, N);
+    else add_runs_kernel<float><<<grid, 256, 0, st>>>((const float*)workspace, k_splits, stride, (float*)Y, ldy, M, N);
+    SP_LAUNCH_CHECK("add_runs");
+    return 0;
 }
 
 // W in operand order (see above), every group N (2N with GLU) rows of K.

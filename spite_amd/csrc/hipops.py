@@ -48,6 +48,7 @@ def lib():
             "spite_attn_decode": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, P],
             "spite_gemm_mfma": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, P],
             "spite_gemm_tiled": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, P],
+            "spite_gemm_tiled_split": [P, I, P, P, I, I, I, I, I, I, P, P],
             "spite_attn_prefill": [P, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, F, I, P],
             "spite_argmax_rows": [P, I, I, I, P, P, P, P],
         }
@@ -399,6 +400,18 @@ def operand_order(w: torch.Tensor) -> torch.Tensor:
     return t.contiguous().view(*lead, N, K)
 
 
+def tiled_k_runs(M: int, N: int, K: int) -> int:
+    """Into how many runs the tiled product cuts its sum over k: with fewer than 128 tiles of
+    128 rows x 512 columns the chip's 256 CUs are not filled, and a run keeps at least four steps
+    of 64 k."""
+    tiles = -(-M // 128) * -(-N // 512)
+    steps = K // 64
+    runs = min(8, 256 // max(tiles, 1), steps // 4)
+    while runs > 1 and -(-steps // runs) * (runs - 1) >= steps:      # no run may be empty
+        runs -= 1
+    return runs if tiles < 128 and runs > 1 else 1
+
+
 def gemm_tiled(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None, glu=False,
                shape=0):
     """Tiled bf16 MFMA product for many rows over weights in operand order (``operand_order``;
@@ -406,6 +419,15 @@ def gemm_tiled(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_sca
     rows_w = _gemm_checks(a, w, y, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, "gemm_tiled")
     if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise KernelError(f"gemm_tiled: bfloat16 operands only, got {a.dtype} and {w.dtype}")
+    runs = tiled_k_runs(M, N, K) if (offsets is None and a_rows is None and a_scale is None and y_rows is None
+                                     and not glu and shape == 0 and M > 0) else 1
+    if runs > 1:
+        # few tiles (a short prompt against a narrow matrix): the sum over k is cut into runs,
+        # each a workgroup of its own, and their partial sums are added by a second kernel
+        part = torch.empty((runs, M, N), dtype=torch.float32, device=a.device)
+        _check(lib().spite_gemm_tiled_split(_ptr(a, "a"), a.stride(0), _ptr(w, "w"), _ptr(y, "y"), dtype_code(y.dtype),
+                                            y.stride(0), M, N, K, runs, _ptr(part, "part"), _stream()), "gemm_tiled")
+        return
     _check(lib().spite_gemm_tiled(
         _ptr(a, "a"), a.stride(0), _ptr(w, "w"), rows_w * K, _ptr(y, "y"), dtype_code(y.dtype), y.stride(0),
         M, N, K, _ptr(offsets, "offsets", torch.int32, True), n_groups, _ptr(a_rows, "a_rows", torch.int32, True),

@@ -243,6 +243,20 @@ def test_gemm_over_many_groups(M, groups, glu):
             run_gemm(ops().gemm_skinny, torch.bfloat16, torch.float32, M, N, K, glu, True, groups=groups, variant=variant)
 
 
+@pytest.mark.parametrize("M,N,K", [(100, 512, 1024), (256, 1040, 2048), (70, 64, 4096), (300, 528, 320), (1, 16, 512)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_gemm_tiled_with_the_sum_over_k_cut_into_runs(M, N, K, out_dtype):
+    """Few tiles: the wrapper cuts k into runs (also runs of unequal length) and adds them up."""
+    from spite_amd.csrc.hipops import tiled_k_runs
+    runs = tiled_k_runs(M, N, K)
+    assert runs > 1 or K < 512, (M, N, K, runs)
+    assert tiled_k_runs(2048, 7168, 5120) == 1          # enough tiles: one run
+
+    def fn(a, w, y, *args, **kw):
+        ops().gemm_tiled(a, ops().operand_order(w), y, *args, **kw)
+    run_gemm(fn, torch.bfloat16, out_dtype, M, N, K)
+
+
 def test_gemm_tiled_refuses_what_it_cannot_do():
     from spite_amd.csrc.hipops import KernelError
     a, w, y = rnd(4, 96, dtype=torch.bfloat16), rnd(32, 96, dtype=torch.bfloat16), rnd(4, 32)
