@@ -262,7 +262,8 @@ def main() -> int:
         log(f"decode batch {b}: {d_b / n * 1e3:.2f} ms/step")
 
     out = {
-        "metric": f"decode tok/s at batch {args.batch}, context {args.context} (Llama 4 Scout shape, random weights)",
+        "metric": f"decode tok/s at batch {args.batch}, context {args.context} "
+                  f"({'a tiny Llama 4 shape' if args.tiny else 'Llama 4 Scout shape'}, random weights)",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic: random weights N(0,0.02), uniform-random token ids, "
