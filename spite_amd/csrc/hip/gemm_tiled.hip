@@ -176,6 +176,36 @@ void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restri
             step(w0, w1, w2, u);
             if (u + 1 < nu) step(w2, w0, w1, u + 1);
         }
+    } else if constexpr (NB == 4) {
+        // few slots a wave (short prompts, where the time is the stream of W from memory): the
+        // accumulators' registers go to six sets of W, each asked for again as soon as its
+        // products are issued, five half steps ahead of its use: three times the bytes in flight
+        bf16x8 w3[4], w4[4], w5[4];
+        auto step6 = [&](bf16x8 (&wa)[4], bf16x8 (&wb)[4], int u) {
+            load_x(xr, u + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            mul(wa, u & 1, 0);
+            load_w(wa, 2 * u + 6);
+            __builtin_amdgcn_sched_barrier(0);
+            mul(wb, u & 1, 1);
+            load_w(wb, 2 * u + 7);
+            store_x(xr, (u + 1) & 1);
+            __syncthreads();
+        };
+        load_x(xr, 0);
+        load_w(w0, 0); load_w(w1, 1); load_w(w2, 2); load_w(w3, 3); load_w(w4, 4); load_w(w5, 5);
+        store_x(xr, 0);
+        __syncthreads();
+        int u = 0;
+        for (; u + 3 <= nu; u += 3) {
+            step6(w0, w1, u);
+            step6(w2, w3, u + 1);
+            step6(w4, w5, u + 2);
+        }
+        if (u < nu) {
+            step6(w0, w1, u);
+            if (u + 1 < nu) step6(w2, w3, u + 1);
+        }
     } else {
         // more slot tiles a wave: the registers of the third set go to the accumulators, and a
         // set is asked for again as soon as its products are issued, one half step ahead
@@ -311,7 +341,9 @@ extern "C" int spite_gemm_tiled_split(const void* X, int ldx, const void* W, voi
 
 // W in operand order (see above), every group N (2N with GLU) rows of K.
 // `shape`: 0 lets the library choose; 1 = 512 W rows x 128 slots a workgroup, 2 = 256 x 256,
-// 3 = 512 x 160 (for groups of a little over 128 rows, which would need a second tile of 128).
+// 3 = 512 x 160 (for groups of a little over 128 rows, which would need a second tile of 128),
+// 4 and 5 = 512 x 64 with W asked for five half steps ahead (short prompts: the stream of W from
+// memory is the time; 4 reads W with non-temporal loads, 5 with plain ones).
 extern "C" int spite_gemm_tiled(const void* X, int ldx, const void* W, long w_group_stride, void* Y, int y_dtype,
                                 int ldy, int M, int N, int K, const int* offsets, int n_groups, const int* a_rows,
                                 const float* a_scale, const int* y_rows, int glu, int shape, hipStream_t st) {
@@ -321,11 +353,23 @@ extern "C" int spite_gemm_tiled(const void* X, int ldx, const void* W, long w_gr
     SP_REQUIRE(((uintptr_t)X & 15) == 0 && ((uintptr_t)W & 15) == 0, "gemm_tiled: operands must be 16-byte aligned");
     SP_REQUIRE(y_dtype == SP_BF16 || y_dtype == SP_F32, "gemm_tiled: output dtype %d", y_dtype);
     SP_REQUIRE(!offsets || n_groups > 0, "gemm_tiled: grouped call without groups");
-    SP_REQUIRE(shape >= 0 && shape <= 3, "gemm_tiled: tile shape %d", shape);
+    SP_REQUIRE(shape >= 0 && shape <= 5, "gemm_tiled: tile shape %d", shape);
     if (M == 0) return 0;
     if (shape == 0) shape = 1;          // measured the faster one at every shape of Llama 4 Scout
     if (shape == 1)
         return launch_tiled<8, 1, 8>(X, ldx, W, w_group_stride, Y, y_dtype, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, st);
+    if (shape == 4 || shape == 5) {
+        // 512 x 64, six W sets ahead: 4 streams W with non-temporal loads, 5 with plain ones
+#define SP_T4(GLUV, TY, NTV) launch_tiled_kernel<8, 1, 4, GLUV, TY, NTV>(X, ldx, W, w_group_stride, Y, ldy, M, N, K, offsets, \
+                                                                     n_groups, a_rows, a_scale, y_rows, 1, 0, st)
+        if (shape == 4) {
+            if (glu) return y_dtype == SP_BF16 ? SP_T4(true, bf16, true) : SP_T4(true, float, true);
+            return y_dtype == SP_BF16 ? SP_T4(false, bf16, true) : SP_T4(false, float, true);
+        }
+        if (glu) return y_dtype == SP_BF16 ? SP_T4(true, bf16, false) : SP_T4(true, float, false);
+        return y_dtype == SP_BF16 ? SP_T4(false, bf16, false) : SP_T4(false, float, false);
+#undef SP_T4
+    }
     if (shape == 3)
         return launch_tiled<8, 1, 10>(X, ldx, W, w_group_stride, Y, y_dtype, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, st);
     return launch_tiled<4, 2, 8>(X, ldx, W, w_group_stride, Y, y_dtype, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, st);

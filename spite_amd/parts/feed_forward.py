@@ -121,7 +121,8 @@ class MoeTop1Sigmoid(FeedForward):
         # slot s writes row dst[s]: rows [0,T) the routed result per token, rows [T,2T) the shared one
         y = ws.take((2 * T, d), torch.float32)
         # (the down product has too few column tiles for the larger row tile to pay)
-        linear(act, self.w_down, y, offsets=offsets, n_groups=groups, y_rows=dst, rows=n, max_rows=T)
+        linear(act, self.w_down, y, offsets=offsets, n_groups=groups, y_rows=dst, rows=n, max_rows=T,
+               tile_shape=shape if shape == 4 else 0)
         if self.fused_shared:
             return (y[:T], y[T:])
         act_s = ws.take((T, self.Fs), x.dtype)

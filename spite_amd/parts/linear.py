@@ -41,14 +41,23 @@ class Weight:
 def grouped_tile_shape(tokens: int, groups: int, whole_groups: int = 0) -> int:
     """Which tile of the prefill product suits ``tokens`` rows that spread evenly over ``groups``
     groups (experts that a router picks), beside ``whole_groups`` groups that take every row.
-    A group costs whole row tiles, each of which streams the group's weights once: with 128
-    rows a tile (shape 1) half of the groups of about 128 rows need a second tile, with 160
-    (shape 3, about a sixth dearer per tile) almost none.  The expected number of tiles of
-    each shape decides, group sizes taken as normal around tokens/groups."""
+    A group costs whole row tiles, each of which streams the group's weights once.
+
+    * Few rows a group and few groups (a short prompt over a few experts): the time is the stream
+      of the weights from memory and there are too few workgroups to keep it busy; the 64-row
+      tile with its deeper run of loads (shape 4) streams faster, as long as the groups that take
+      every row do not need many of those small tiles.  (With 128 experts there are workgroups
+      enough: measured no gain.)
+    * Else 128 rows a tile (shape 1), or 160 (shape 3, about a sixth dearer per tile) where that
+      saves tiles: with groups of about 128 rows half of them need a second tile of 128, almost
+      none a second one of 160.  The expected number of tiles of each shape decides, group sizes
+      taken as normal around tokens/groups."""
     if groups <= 0 or tokens <= 0:
         return 1
     mean = tokens / groups
     sd = max(math.sqrt(tokens * (1.0 / groups) * (1.0 - 1.0 / groups)), 1e-6)
+    if groups <= 32 and mean + 4.0 * sd <= 64.0 and whole_groups * -(-tokens // 64) <= 0.25 * groups:
+        return 4
 
     def tiles(rows_per_tile):
         extra, k = 0.0, 1

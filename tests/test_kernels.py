@@ -215,7 +215,7 @@ def test_gemm_skinny_over_operand_order(M, N, K, out_dtype, glu, grouped, varian
                                                   (300, 64, 448)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("glu,grouped", [(False, False), (True, False), (False, True), (True, True)])
-@pytest.mark.parametrize("shape", [1, 2, 3])
+@pytest.mark.parametrize("shape", [1, 2, 3, 4, 5])
 def test_gemm_tiled(M, N, K, out_dtype, glu, grouped, shape):
     def fn(a, w, y, *args, **kw):
         ops().gemm_tiled(a, ops().operand_order(w), y, *args, **kw)
@@ -233,7 +233,7 @@ def test_gemm_over_many_groups(M, groups, glu):
 
     def tiled(a, w, y, *args, **kw):
         ops().gemm_tiled(a, ops().operand_order(w), y, *args, **kw)
-    for shape in (1, 3):
+    for shape in (1, 3, 4):
         run_gemm(tiled, torch.bfloat16, torch.float32, M, N, K, glu, True, groups=groups, shape=shape)
     if M <= 64:
         for variant in (2, 8, 9):
