@@ -11,15 +11,20 @@
 // band follow each other in k, so a wave streams its four bands.
 //
 // A workgroup of eight waves owns 16*NB*WM rows of X ("slots") and 64*WN rows of W
-// (WN * WM = 8); a wave owns 64 rows of W and 16*NB slots: 4 x NB accumulator tiles (NB = 8,
-// or 10 where the registers of the third W set go to the accumulators).
+// (WN * WM = 8); a wave owns 64 rows of W and 16*NB slots: 4 x NB accumulator tiles (NB = 8;
+// 10 where the registers of the third W set go to the accumulators; 4 for short prompts, where
+// the accumulators' registers go to more W sets).
 //  * W never touches LDS: three rotating sets of operand registers, loaded two steps of 32 k
-//    ahead of the products (NB = 10: two sets, one step ahead).
+//    ahead of the products (NB = 10: two sets, one step ahead; NB = 4: six sets, five ahead).
+//    NTW: W is read with non-temporal loads (where a band of W meets few row tiles it is read
+//    once, and such a stream runs faster past the caches).
 //  * X is the "B" operand, shared by the waves: tiles of 64 k go through LDS, fetched with
 //    eight lanes a row (whole cache lines), rows padded by 16 bytes against bank conflicts,
 //    double-buffered, one barrier per 64 k.
 //  * Tiles are handed out so that the workgroups running on one XCD (one L2) at a time share
 //    W bands and walk K together.
+//  * k_splits > 1: a tile's sum over k is cut into runs, each a workgroup of its own that
+//    writes partial sums (plain products over few tiles; the caller adds the runs).
 // Grouped form (experts) and GLU as in gemm_generic.hip; with GLU a wave's bands are two of
 // gate rows and the two matching of up rows.
 #include "common.h"
