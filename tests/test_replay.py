@@ -202,6 +202,30 @@ def test_schedules_agree_with_each_other(case):
         assert d <= case.tol, f"{k} differs from whole by {d} at {where}"
 
 
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_other_mixed_schedules_agree_with_whole(case, seed):
+    """More ways of cutting and mixing the same requests, also with portions of 31 and 64 tokens
+    (a page's edge, a chunk's edge, several pages in one portion), against the whole replay;
+    in bfloat16 with the whole replay's experts."""
+    if "whole" not in case.results:
+        pytest.skip("the whole replay failed")
+    ps = PAGE[case.name]
+    pool = sum(sorted((-(-len(t) // ps) * ps for t in case.reqs.values()), reverse=True)[:4])
+    steps = H.schedule_mixed(case.reqs, seed=seed, portion_sizes=(2, 3, 5, 8, 13, 31, 64))
+    take = None
+    if case.dtype != "float32":
+        whole_steps = H.schedule_whole(case.reqs)
+        if not hasattr(case, "whole_hints"):
+            case.whole_rows, case.whole_hints = case.replay(whole_steps, case.pool)
+        take = H.experts_to_take(case.cfg, steps, case.whole_hints)
+    rows, _ = case.replay(steps, pool, take=take)
+    want = case.results["whole"] if case.dtype == "float32" else case.whole_rows
+    d, where = H.max_diff(rows, want)
+    tol = TOL_F32_SCHEDULES if case.dtype == "float32" else case.tol
+    print(f"[{case.name} {case.dtype}] mixed schedule {seed} vs whole: {d:.3e} (tol {tol:.3e})")
+    assert d <= tol, f"schedule {seed} differs from whole by {d} at {where}"
+
+
 def test_first_tokens_of_a_sequence(case):
     # one-token and two-token requests, and position 0 of every request
     first = case.reqs[next(iter(case.reqs))]
