@@ -17,3 +17,35 @@ def test_tile_shape_follows_the_expected_number_of_row_tiles():
     assert grouped_tile_shape(3200, 16, 1) == 1
     # nothing to spread
     assert grouped_tile_shape(0, 16, 1) == 1 and grouped_tile_shape(100, 0) == 1
+
+
+def test_runs_of_a_split_product_are_never_empty():
+    from spite_amd.csrc.hipops import tiled_k_runs
+    for M in (65, 100, 256, 700, 2048):
+        for N in (16, 512, 5120, 7168, 202048):
+            for K in (64, 192, 320, 1024, 5120, 8192):
+                runs, steps = tiled_k_runs(M, N, K), K // 64
+                assert 1 <= runs <= 8
+                if runs > 1:
+                    per = -(-steps // runs)
+                    assert per * (runs - 1) < steps and per >= 4 and -(-M // 128) * -(-N // 512) < 128
+
+
+def test_the_benchmark_counts_what_a_query_can_see():
+    import importlib.util
+    import os
+    spec = importlib.util.spec_from_file_location("bench", os.path.join(os.path.dirname(os.path.dirname(__file__)), "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    for T, past, span in ((5, 0, None), (7, 9, None), (6, 0, 4), (10, 13, 8), (3, 7, 8), (20, 30, 16)):
+        brute = sum(1 for p in range(past, past + T) for j in range(p + 1) if span is None or j >= (p // span) * span)
+        assert bench.visible_pairs(T, past, span) == brute
+    cfg = dict(bench.SCOUT)
+    # more context costs more bytes on every layer below a chunk, only on every fourth above it
+    a = bench.decode_bytes(cfg, 48, 8, 4096, 6.4)
+    b = bench.decode_bytes(cfg, 48, 8, 4097, 6.4)
+    c = bench.decode_bytes(cfg, 48, 8, 32768, 6.4)
+    d = bench.decode_bytes(cfg, 48, 8, 32769, 6.4)
+    kv_token = 2 * 8 * 128 * 2
+    assert b - a == 8 * 48 * kv_token and d - c == 8 * 48 * kv_token
+    assert bench.decode_bytes(cfg, 48, 8, 8192, 6.4) < bench.decode_bytes(cfg, 48, 8, 8191, 6.4)   # a new chunk begins
