@@ -97,8 +97,7 @@ void attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_p
                 s[tt][i] = v;
                 mx = fmaxf(mx, v);
             }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        mx = rows4_max(mx);
         const float m_new = fmaxf(m_run, mx);
         const float alpha = (m_run == -INFINITY) ? 0.f : exp2f(m_run - m_new);
         float sum = 0.f;
@@ -111,8 +110,7 @@ void attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_p
                 sum += e;
                 pf[tt * 4 + i] = (bf16)e;
             }
-        sum += __shfl_xor(sum, 16, 64);
-        sum += __shfl_xor(sum, 32, 64);
+        sum = rows4_sum(sum);
         l_run = l_run * alpha + sum;
         m_run = m_new;
 #pragma unroll
