@@ -1,7 +1,6 @@
 """ctypes binding of the host runtime library (cache manager, scheduler)."""
 from __future__ import annotations
 
-import ctypes
 from ctypes import c_int, c_longlong, c_ulonglong, c_void_p, c_char_p, POINTER
 
 from . import build

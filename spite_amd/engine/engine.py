@@ -8,15 +8,14 @@ fp32 logits at the wanted places.  The reference's ``forward(tokens, logits_out,
 """
 from __future__ import annotations
 
-import json
 import os
-from dataclasses import dataclass, field
-from typing import Dict, List, Optional, Sequence, Union
+from dataclasses import dataclass
+from typing import Dict, Optional, Sequence, Union
 
 import numpy as np
 import torch
 
-from ..cache.paged import PagedCache, CacheError, OutOfPages
+from ..cache.paged import PagedCache
 from ..config import read_config
 from ..csrc import hipops
 from ..parts.base import ModelSpec, LayerCall

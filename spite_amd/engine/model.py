@@ -10,7 +10,7 @@ from ..csrc import hipops
 from ..parts import base as P
 from ..parts.base import ParamSpec, PartSpec, CacheNeed
 from ..parts.linear import linear, Weight
-from .context import Env, Workspace, StepContext, LayerCache
+from .context import Env, Workspace, StepContext
 
 
 class Model:

@@ -6,7 +6,6 @@ import ctypes
 from dataclasses import dataclass
 from typing import List, Sequence
 
-import numpy as np
 
 from ..csrc import hostlib
 

@@ -11,11 +11,11 @@ float32 run everything is widened to fp32.
 """
 from __future__ import annotations
 
-from typing import Dict, List
+from typing import Dict
 
 import torch
 
-from .safetensors_io import Checkpoint, SafetensorsError
+from .safetensors_io import Checkpoint
 
 PREFIXES = ("language_model.",)
 

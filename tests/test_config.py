@@ -1,7 +1,6 @@
 """Configuration: reading config.json keys into the typed configuration, one error that
 lists every problem, the architecture registry, the layer list that the spec derives."""
 import json
-import os
 
 import pytest
 

@@ -3,7 +3,6 @@ replay, with the program's own eager work (prefill steps of other shapes, new re
 between the replays."""
 import numpy as np
 import pytest
-import torch
 
 import helpers as H
 

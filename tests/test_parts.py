@@ -2,7 +2,6 @@
 activations, outside any model, and compared with the plain implementation's function for
 that part.  Mixers are stepped twice on one request (a portion, then another) so that the
 second call reads what the first left in the cache."""
-import math
 
 import numpy as np
 import pytest

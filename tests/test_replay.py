@@ -5,7 +5,6 @@ each other.  The logits at a position must not depend on how the tokens were cut
 steps, on what else was in the batch, or on which pages were used."""
 import numpy as np
 import pytest
-import torch
 
 import helpers as H
 

@@ -3,10 +3,8 @@ size is defined here, registered, put into a model beside the built-in attention
 stepped - whole, token by token and in portions, several requests in a batch - without a
 change to the framework's files.  The layer order is data: one block runs twice (on caches
 of its own), and one attention layer reads the cache that another layer wrote."""
-import numpy as np
 import pytest
 import torch
-import torch.nn.functional as F
 
 import helpers as H
 
