@@ -208,7 +208,10 @@ extern "C" int spite_gemm_skinny(const void* X, int ldx, const void* W, long w_g
         // (groups of experts at 33 to 64 tokens hold a few rows each, only the shared one all:
         // 32 columns a workgroup and a second row tile for that group beat 64 columns for all)
         else if (offsets) variant = glu ? 2 : 10;
-        else variant = 9;
+        // (a plain product's time grows with the tokens, whose rows every workgroup reads from
+        // L2 beside its rows of W: from about 50 tokens on, 64 rows of W a workgroup with two row
+        // tiles of 32 columns beat 32 rows of W with all 64 columns)
+        else variant = max_rows > 48 ? 10 : 9;
     }
     switch (variant) {
         case 2: return launch_skinny<2, 2, 2, 8>(SP_ARGS);
