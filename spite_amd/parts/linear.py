@@ -37,6 +37,13 @@ class Weight:
                           and w.shape[-2] % 16 == 0 and w.shape[-1] % 64 == 0)
         self.data = hipops.operand_order(w) if self.tiled else w
 
+    def group(self, g: int) -> "Weight":
+        """Group ``g`` of a stack of matrices ``[groups, out, in]`` as a weight of its own (the same
+        memory)."""
+        one = object.__new__(Weight)
+        one.data, one.tiled, one.shape, one.dtype = self.data[g], self.tiled, self.shape[1:], self.dtype
+        return one
+
 
 def grouped_tile_shape(tokens: int, groups: int, whole_groups: int = 0) -> int:
     """Which tile of the prefill product suits ``tokens`` rows that spread evenly over ``groups``

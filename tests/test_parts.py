@@ -172,6 +172,37 @@ def test_moe_reference_vector_through_the_part():
         assert abs(y[0] - 30.0) < 0.2 and abs(y[1] - 60.0) < 0.4 and y[2:].abs().max() == 0
 
 
+@pytest.mark.parametrize("T", [9, 32, 33, 48, 64, 65, 150])
+def test_experts_with_weights_in_operand_order(T):
+    """The experts' part alone at sizes whose weights lie in MFMA operand order (the tiny
+    configurations' do not), over the token counts at which it changes its products: few rows
+    (one grouped product), 33 to 64 (the shared expert as a product of its own), more (tiles)."""
+    from spite_amd.engine.context import Env, Workspace, StepContext, HostBatch
+    from spite_amd.parts.feed_forward import MoeTop1Sigmoid
+    d, F_, E = 128, 64, 16
+    g = torch.Generator().manual_seed(100 + T)
+    rnd = lambda *s, std=1.0: torch.randn(*s, generator=g) * std
+    w = {"router": rnd(E, d, std=0.5), "experts.gate_up_proj": rnd(E, d, 2 * F_, std=0.1),
+         "experts.down_proj": rnd(E, F_, d, std=0.1), "shared.gate_proj": rnd(F_, d, std=0.1),
+         "shared.up_proj": rnd(F_, d, std=0.1), "shared.down_proj": rnd(d, F_, std=0.1)}
+    w = {k: (v if k == "router" else v.to(torch.bfloat16)) for k, v in w.items()}
+    part = MoeTop1Sigmoid(Env(torch.bfloat16, torch.device(DEV)), hidden_size=d, intermediate_size=F_, n_experts=E)
+    part.load({k: v.to(DEV) for k, v in w.items()})
+    assert part.w_gate_up.tiled and part.w_down.tiled
+    x = rnd(T, d).to(torch.bfloat16)
+    ctx = StepContext(T=T, n_seqs=1, token_ids=None, positions=None, seq_of_token=None, cu_seqlens=None,
+                      seq_slots=None, seq_starts=None, logit_rows=None, n_out=0,
+                      host=HostBatch(np.zeros(1), np.zeros(1), np.full(1, T), np.array([0, T])),
+                      ws=Workspace(torch.device(DEV), 1 << 24))
+    outs = part.forward(x.to(DEV), x.to(DEV).float(), ctx)
+    W = {k: v.double() for k, v in w.items()}
+    ref = plain.moe_ffn(x.double(), W["router"], W["experts.gate_up_proj"], W["experts.down_proj"],
+                        W["shared.gate_proj"], W["shared.up_proj"], W["shared.down_proj"])
+    got = sum(o.double() for o in outs).cpu()
+    err = (got - ref).abs().max().item()
+    assert err <= 1e-2 * ref.abs().max().item(), (T, err, ref.abs().max().item())
+
+
 def test_block_alone(rig):
     from spite_amd.parts.base import LayerCall
     cfg, W = rig.cfg, rig.w
