@@ -294,8 +294,6 @@ class Engine:
             if toks.min() < 0 or toks.max() >= V:
                 bad = int(toks[(toks < 0) | (toks >= V)][0])
                 raise EngineError(f"entry {i}: token id {bad} outside the vocabulary of {V}")
-            if self.cache.cached(e.slot) + len(e.tokens) > self.spec.max_position:
-                raise EngineError(f"entry {i}: position beyond the model's limit {self.spec.max_position}")
             total += len(e.tokens)
         for e in entries:
             self.cache.reserve(e.slot, len(e.tokens))

@@ -81,7 +81,7 @@ class ModelSpec:
     embed_name: str
     head_name: Optional[str]     # None: the embedding table is the output matrix
     eos_token_ids: Tuple[int, ...] = ()
-    max_position: int = 1 << 20
+    max_position: int = 1 << 20  # the default context limit of generation (the step function itself has none)
 
 
 class Part:

@@ -239,6 +239,21 @@ def test_long_decoding(case):
     check(case, case.replay(H.schedule_tail_one_by_one(reqs, tail=150), 160), "long decode", reqs)
 
 
+def test_the_step_has_no_context_limit(tmp_path):
+    """``max_position_embeddings`` bounds what generation is asked for, not what a step runs:
+    a replay that goes past it gives the plain implementation's logits."""
+    from spite_amd.engine.engine import Engine
+    cfg = dict(H.CONFIGS["A"], max_position_embeddings=32)
+    folder = str(tmp_path / "short_limit")
+    weights = H.make_model(folder, cfg, seed=9, dtype="float32")
+    reqs = {"x": H.random_tokens(cfg["vocab_size"], 75, 3)}
+    steps = H.schedule_portions(reqs)
+    eng = Engine(folder, dtype="float32", page_size=16, cache_tokens=128, max_requests=2)
+    rows = H.collect(steps, H.run_trace_inprocess(eng, steps), cfg["vocab_size"])
+    d, where = H.max_diff(rows, H.plain_logits(cfg, weights, reqs))
+    assert d <= TOL_F32, (d, where)
+
+
 def test_trace_run_program(case):
     """The program itself, as a user runs it: page size 64, the pool given by --max-tokens."""
     reqs = dict(list(case.reqs.items())[:3])
