@@ -102,7 +102,8 @@ extern "C" int spite_gemm_generic(const void* A, int lda, const void* W, long w_
                M, N, K, lda, ldy);
     SP_REQUIRE(!offsets || n_groups > 0, "gemm: grouped call without groups");
     if (M == 0) return 0;
-    const int m_tiles = (M + GBM - 1) / GBM + (offsets ? n_groups : 0);
+    // row tiles: a group with rows has 1 + (rows - 1) / tile of them, so groups with rows + M / tile bounds them
+    const int m_tiles = offsets ? M / GBM + (n_groups < M ? n_groups : M) : (M + GBM - 1) / GBM;
     SP_REQUIRE(m_tiles <= 65535, "gemm: too many row tiles (%d)", m_tiles);
     dim3 grid((N + GBN - 1) / GBN, m_tiles);
 #define SP_GEMM_LAUNCH(T, TY, GLU) gemm_generic_kernel<T, TY, GLU><<<grid, 256, 0, st>>>( \

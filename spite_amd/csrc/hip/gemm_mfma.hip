@@ -185,7 +185,8 @@ static int launch_mfma(const void* X, int ldx, const void* W, long w_group_strid
                        int N, int K, const int* offsets, int n_groups, const int* a_rows, const float* a_scale,
                        const int* y_rows, int glu, hipStream_t st) {
     constexpr int BM = 128 * WM, BN = 64 * WN;
-    const int m_tiles = (M + BM - 1) / BM + (offsets ? n_groups : 0);
+    // row tiles: a group with rows has 1 + (rows - 1) / tile of them, so groups with rows + M / tile bounds them
+    const int m_tiles = offsets ? M / BM + (n_groups < M ? n_groups : M) : (M + BM - 1) / BM;
     const int ncols = glu ? BN / 2 : BN;
     const int n_tiles = (N + ncols - 1) / ncols;
     SP_REQUIRE((long)m_tiles * n_tiles < (1L << 30), "gemm_mfma: too many tiles");

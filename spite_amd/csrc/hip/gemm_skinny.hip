@@ -162,9 +162,14 @@ void gemm_skinny_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restr
 template <int R, int G, int S, int NW>
 static int launch_skinny(const void* X, int ldx, const void* W, long wgs, void* Y, int y_dtype, int ldy, int M, int N,
                          int K, const int* offsets, int n_groups, const int* a_rows, const float* a_scale,
-                         const int* y_rows, int glu, int tiled, hipStream_t st) {
+                         const int* y_rows, int glu, int tiled, int live_groups, hipStream_t st) {
     const int MT = 16 * G;
-    const int m_tiles = (M + MT - 1) / MT + (offsets ? n_groups : 0);
+    // row tiles: a group with rows has 1 + (rows - 1) / MT of them, so (groups with rows) + M / MT bounds them.
+    // A workgroup of a tile that does not exist leaves at once, but only after it was given its registers:
+    // with 128 groups of which 2 hold rows those were two thirds of the kernel's time.
+    int live = n_groups < M ? n_groups : M;
+    if (live_groups > 0 && live_groups < live) live = live_groups;
+    const int m_tiles = offsets ? M / MT + live : (M + MT - 1) / MT;
     SP_REQUIRE(m_tiles <= 65535, "gemm_skinny: too many row tiles (%d)", m_tiles);
     dim3 grid((N + 16 * R - 1) / (16 * R), m_tiles);
     const size_t sh = (size_t)NW * (glu ? 2 : 1) * R * G * 4 * 64 * sizeof(float);
@@ -182,11 +187,12 @@ static int launch_skinny(const void* X, int ldx, const void* W, long wgs, void* 
 }
 
 // `max_rows`: the most rows any group brings (M itself for a plain product); picks how many
-// token columns a workgroup carries.
+// token columns a workgroup carries.  `live_groups`: the caller's promise that no more groups than
+// this hold rows (0: no promise); the grid is cut to the row tiles that can exist.
 extern "C" int spite_gemm_skinny(const void* X, int ldx, const void* W, long w_group_stride, void* Y, int y_dtype,
                                  int ldy, int M, int N, int K, const int* offsets, int n_groups, const int* a_rows,
                                  const float* a_scale, const int* y_rows, int glu, int max_rows, int variant,
-                                 int w_tiled, hipStream_t st) {
+                                 int w_tiled, int live_groups, hipStream_t st) {
     SP_REQUIRE(M >= 0 && N > 0 && K > 0 && ldx >= K && ldy >= N, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
     SP_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "gemm_skinny: K=%d and the row stride %d must be multiples of 8", K, ldx);
     SP_REQUIRE(((uintptr_t)X & 15) == 0 && ((uintptr_t)W & 15) == 0, "gemm_skinny: operands must be 16-byte aligned");
@@ -194,7 +200,7 @@ extern "C" int spite_gemm_skinny(const void* X, int ldx, const void* W, long w_g
     SP_REQUIRE(!offsets || n_groups > 0, "gemm_skinny: grouped call without groups");
     SP_REQUIRE(!w_tiled || (K % 32 == 0 && N % 16 == 0), "gemm_skinny: operand order needs K=%d a multiple of 32 and N=%d of 16", K, N);
     if (M == 0) return 0;
-#define SP_ARGS X, ldx, W, w_group_stride, Y, y_dtype, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, w_tiled, st
+#define SP_ARGS X, ldx, W, w_group_stride, Y, y_dtype, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, w_tiled, live_groups, st
     // measured on MI355X (GB/s of W at Llama 4 Scout's shapes): one row tile per workgroup for
     // the experts' grouped stream, two for the dense projections, four for the output matrix
     if (variant == 0) {

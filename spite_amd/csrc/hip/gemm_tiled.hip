@@ -269,7 +269,8 @@ static int launch_tiled_kernel(const void* X, int ldx, const void* W, long w_gro
                                int K, const int* offsets, int n_groups, const int* a_rows, const float* a_scale,
                                const int* y_rows, int k_splits, size_t split_stride, hipStream_t st) {
     constexpr int BM = 16 * NB * WM, BN = 64 * WN;
-    const int m_tiles = (M + BM - 1) / BM + (offsets ? n_groups : 0);
+    // row tiles: a group with rows has 1 + (rows - 1) / tile of them, so groups with rows + M / tile bounds them
+    const int m_tiles = offsets ? M / BM + (n_groups < M ? n_groups : M) : (M + BM - 1) / BM;
     const int ncols = GLU ? BN / 2 : BN;
     const int n_tiles = (N + ncols - 1) / ncols;
     SP_REQUIRE((long)m_tiles * n_tiles * k_splits < (1L << 30), "gemm_tiled: too many tiles");

@@ -44,7 +44,7 @@ def lib():
             "spite_attn_generic": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, I, P],
             "spite_sample_rows": [P, I, I, I, P, P, P, P],
             "spite_filter_rows": [P, I, I, I, P, P, P, P],
-            "spite_gemm_skinny": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, I, I, P],
+            "spite_gemm_skinny": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, I, I, I, P],
             "spite_attn_decode": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, P],
             "spite_gemm_mfma": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, P],
             "spite_gemm_tiled": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, P],
@@ -311,10 +311,11 @@ def _gemm_checks(a, w, y, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, g
 
 
 def gemm_skinny(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None,
-                glu=False, max_rows=None, variant=0, tiled=False):
+                glu=False, max_rows=None, variant=0, tiled=False, live_groups=0):
     """Weight-streaming bf16 product for few rows (see gemm_skinny.hip); arguments as gemm_generic.
     ``max_rows``: the most rows a group can bring (default M).  ``tiled``: w is in MFMA operand
-    order (``operand_order``)."""
+    order (``operand_order``).  ``live_groups``: a promise that at most this many groups hold rows
+    (0: none); row tiles beyond what that allows are not launched."""
     rows_w = _gemm_checks(a, w, y, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, "gemm_skinny")
     if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise KernelError(f"gemm_skinny: bfloat16 operands only, got {a.dtype} and {w.dtype}")
@@ -322,7 +323,8 @@ def gemm_skinny(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_sc
         _ptr(a, "a"), a.stride(0), _ptr(w, "w"), rows_w * K, _ptr(y, "y"), dtype_code(y.dtype), y.stride(0),
         M, N, K, _ptr(offsets, "offsets", torch.int32, True), n_groups, _ptr(a_rows, "a_rows", torch.int32, True),
         _ptr(a_scale, "a_scale", torch.float32, True), _ptr(y_rows, "y_rows", torch.int32, True), int(glu),
-        int(max_rows if max_rows is not None else M), int(variant), int(bool(tiled)), _stream()), "gemm_skinny")
+        int(max_rows if max_rows is not None else M), int(variant), int(bool(tiled)), int(live_groups), _stream()),
+        "gemm_skinny")
 
 
 def kv_tiled_ok(dtype, hd, page_size) -> bool:

@@ -137,12 +137,14 @@ class MoeTop1Sigmoid(FeedForward):
             linear(act[T:], self.w_down.group(E), y, y_rows=dst[T:], rows=T)
             return (y[:T], y[T:])
         shape = grouped_tile_shape(T, E, groups - E) if T > SKINNY_MAX_ROWS else 0
+        # every token goes to one expert: at most min(T, E) of their groups hold rows, and the shared one
+        live = min(T, E) + (groups - E)
         linear(x, self.w_gate_up, act, glu=True, offsets=offsets, n_groups=groups, a_rows=src, a_scale=scale, rows=n,
-               max_rows=T, tile_shape=shape)
+               max_rows=T, tile_shape=shape, live_groups=live)
         # slot s writes row dst[s]: rows [0,T) the routed result per token, rows [T,2T) the shared one
         # (the down product has too few column tiles for the larger row tile to pay)
         linear(act, self.w_down, y, offsets=offsets, n_groups=groups, y_rows=dst, rows=n, max_rows=T,
-               tile_shape=shape if shape == 4 else 0)
+               tile_shape=shape if shape == 4 else 0, live_groups=live)
         if self.fused_shared:
             return (y[:T], y[T:])
         act_s = ws.take((T, self.Fs), x.dtype)

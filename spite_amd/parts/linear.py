@@ -76,12 +76,13 @@ def grouped_tile_shape(tokens: int, groups: int, whole_groups: int = 0) -> int:
 
 
 def linear(x, w, y, *, glu=False, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None, rows=None,
-           max_rows=None, tile_shape=0):
+           max_rows=None, tile_shape=0, live_groups=0):
     """y[r] = W . x[r] for ``rows`` rows (default: all of x; for a row list: its length).
 
     With ``glu`` the weight holds gate rows then up rows and y = silu(gate) * up.
     ``max_rows``: the most rows that one group can bring (default: ``rows``).
-    ``tile_shape``: the prefill product's tile (``grouped_tile_shape``), 0 = the library's choice."""
+    ``tile_shape``: the prefill product's tile (``grouped_tile_shape``), 0 = the library's choice.
+    ``live_groups``: a promise that at most this many groups hold rows (0: none)."""
     tiled = False
     if isinstance(w, Weight):
         w, tiled = w.data, w.tiled
@@ -94,7 +95,8 @@ def linear(x, w, y, *, glu=False, offsets=None, n_groups=1, a_rows=None, a_scale
         # streamed faster by the tiled kernel from 33 rows on)
         if most <= SKINNY_MAX_ROWS and not (tiled and most > 32 and offsets is None and N >= 65536):
             hipops.gemm_skinny(x, w, y, M, N, K, offsets=offsets, n_groups=n_groups, a_rows=a_rows,
-                               a_scale=a_scale, y_rows=y_rows, glu=glu, max_rows=most, tiled=tiled)
+                               a_scale=a_scale, y_rows=y_rows, glu=glu, max_rows=most, tiled=tiled,
+                               live_groups=live_groups)
         elif tiled:
             hipops.gemm_tiled(x, w, y, M, N, K, offsets=offsets, n_groups=n_groups, a_rows=a_rows, a_scale=a_scale,
                               y_rows=y_rows, glu=glu, shape=tile_shape)

@@ -236,10 +236,16 @@ def test_gemm_over_many_groups(M, groups, glu):
     for shape in (1, 3, 4):
         run_gemm(tiled, torch.bfloat16, torch.float32, M, N, K, glu, True, groups=groups, shape=shape)
     if M <= 64:
+        # the groups that run_gemm will fill: with the promise that no more hold rows the grid is
+        # cut to the row tiles that can exist, and every row must still be served
+        cuts = [0] + sorted(torch.randint(0, M + 1, (groups - 1,), generator=torch.Generator().manual_seed(M)).tolist()) + [M]
+        live = sum(b > a for a, b in zip(cuts, cuts[1:]))
+        assert 0 < live < groups
         for variant in (2, 8, 9):
             def skinny(a, w, y, *args, **kw):
                 ops().gemm_skinny(a, ops().operand_order(w), y, *args, tiled=True, variant=variant, **kw)
             run_gemm(skinny, torch.bfloat16, torch.float32, M, N, K, glu, True, groups=groups)
+            run_gemm(skinny, torch.bfloat16, torch.float32, M, N, K, glu, True, groups=groups, live_groups=live)
             run_gemm(ops().gemm_skinny, torch.bfloat16, torch.float32, M, N, K, glu, True, groups=groups, variant=variant)
 
 
