@@ -321,7 +321,10 @@ def attention_reference(kv, queries, qs, H, vis, span):
     out = torch.zeros(len(queries), H, kv.hd, dtype=torch.float64)
     for t, (s, p) in enumerate(queries):
         pos = torch.arange(p + 1)
-        mask = plain.visible_mask(pos, vis, span)[p:p + 1]
+        if p < 8192:
+            mask = plain.visible_mask(pos, vis, span)[p:p + 1]
+        else:                        # the whole square would not fit: the query's own row of it
+            mask = (pos >= plain_first(vis, span, p)).view(1, -1)
         out[t] = plain.attention(qs[t:t + 1].double(), kv.k[s][:p + 1].double(), kv.v[s][:p + 1].double(), mask)[0]
     return out
 
@@ -477,6 +480,21 @@ def test_attention_finds_one_far_key_among_thousands(kind):
     # the reference itself puts nearly all the weight on key 77: its output is that key's value
     kv = PagedKV([3000], 2, 128, 64, torch.bfloat16, 0)
     assert (ref[0, 0] - kv.v[0][77][0].double()).abs().max() < 0.05
+    assert (got - ref).abs().max() < 2e-2
+
+
+@pytest.mark.parametrize("kind,vis,span,far,n_splits", [
+    ("decode", "full", 0, 123, 64), ("decode", "full", 0, 20000, 256), ("decode", "chunk", 8192, 32768, 16),
+    ("prefill", "full", 0, 123, 0), ("prefill", "chunk", 8192, 32769, 0)])
+def test_attention_at_forty_thousand_keys(kind, vis, span, far, n_splits):
+    """Positions beyond the real model's first chunk borders, page tables of hundreds of pages: one
+    far key (the first ones of the context, or of the query's chunk) carries the answer."""
+    n = 40000
+    queries = [(0, n - 1)] if kind == "decode" else [(0, p) for p in range(n - 18, n)]
+    t = len(queries) // 2
+    got, ref = run_attention(kind, torch.bfloat16, 4, 1, 128, 64, [n], queries, vis, span, n_splits=n_splits, planted=(t, 0, far))
+    kv = PagedKV([n], 1, 128, 64, torch.bfloat16, 0)
+    assert (ref[t, 0] - kv.v[0][far][0].double()).abs().max() < 0.05
     assert (got - ref).abs().max() < 2e-2
 
 
