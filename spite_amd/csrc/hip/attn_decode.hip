@@ -22,6 +22,7 @@
 // Scores, running maximum and sum, and the output are fp32; P is rounded to bf16 only as an
 // MFMA operand.
 #include "common.h"
+#include "no_alloc.h"
 
 template <int HD>
 __global__ __launch_bounds__(256)
@@ -238,4 +239,44 @@ extern "C" int spite_attn_decode(const void* q, const void* k_pages, const void*
     }
     SP_LAUNCH_CHECK("attn_decode_combine");
     return 0;
+}
+
+// ---- the same call for callers that cannot allocate: the partial results go to an array of
+// the library's own.  In host code `scratch` is only a handle for hipGetSymbolAddress; the
+// address of each GPU's copy is looked up once per device and that pointer is what kernels get.
+static __device__ __align__(256) float scratch[SPITE_ATTN_DECODE_STATIC_FLOATS];
+enum { SP_MAX_DEVICES = 64 };
+static float* g_scratch_ptr[SP_MAX_DEVICES];     // per device, null until its first call
+static hipError_t scratch_of_current_device(float** ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= SP_MAX_DEVICES) return hipErrorInvalidDevice;
+    float* p = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+    if (p == nullptr) {
+        e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        __atomic_store_n(&g_scratch_ptr[dev], p, __ATOMIC_RELEASE);
+    }
+    *ptr = p;
+    return hipSuccess;
+}
+
+extern "C" int spite_attn_decode_static(const void* q, const void* k_pages, const void* v_pages, void* out,
+                                        const int* positions, const int* seq_of_token, const int* block_table,
+                                        int max_blocks, int T, int H, int G, int hd, int page_size, int vis, int span,
+                                        float scale, int n_splits, hipStream_t st) {
+    SP_REQUIRE(T >= 0 && H > 0 && (hd == 64 || hd == 128) && n_splits >= 1 && n_splits <= 256,
+               "attn_decode_static: T=%d H=%d hd=%d splits=%d", T, H, hd, n_splits);
+    const size_t need = n_splits > 1 ? (size_t)T * H * n_splits * (hd + 2) : 0;
+    SP_REQUIRE(need <= (size_t)SPITE_ATTN_DECODE_STATIC_FLOATS,
+               "attn_decode_static: %zu floats of partial results (T=%d H=%d splits=%d hd=%d) exceed the library's %u; "
+               "use fewer splits or spite_attn_decode with a workspace", need, T, H, n_splits, hd,
+               (unsigned)SPITE_ATTN_DECODE_STATIC_FLOATS);
+    float* ptr = nullptr;
+    const hipError_t e = scratch_of_current_device(&ptr);
+    SP_REQUIRE(e == hipSuccess && ptr != nullptr, "attn_decode_static: no address for the scratch array: %s",
+               hipGetErrorString(e));
+    return spite_attn_decode(q, k_pages, v_pages, out, ptr, positions, seq_of_token, block_table, max_blocks, T, H, G,
+                             hd, page_size, vis, span, scale, n_splits, st);
 }

@@ -1,0 +1,81 @@
+"""The decode attention entry point that allocates nothing (``spite_attn_decode_static``,
+declared in csrc/hip/no_alloc.h): called through ctypes, two calls in a row on the same GPU,
+the second with a smaller input, each compared with ``spite_attn_decode`` over a workspace of
+the caller's.  Both run the same kernels, so the outputs are equal bit for bit."""
+import ctypes
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+STATIC_FLOATS = 4 << 20
+
+
+def _case(T, H, G, hd, ps, ctx_len, seed):
+    """Random queries and operand-order pages of T requests of ``ctx_len`` keys each."""
+    from spite_amd.csrc import hipops
+    g = torch.Generator().manual_seed(seed)
+    blocks = -(-ctx_len // ps)
+    n_pages = T * blocks + 1
+    kp = torch.randn(n_pages, G, ps, hd, generator=g).to(torch.bfloat16).to(DEV)
+    vp = torch.randn(n_pages, G, hd, ps, generator=g).to(torch.bfloat16).to(DEV)
+    kp, vp = hipops.kv_operand_order(kp, vp)
+    q = torch.randn(T, H * hd, generator=g).to(torch.bfloat16).to(DEV)
+    # request t owns pages 1 + t*blocks ..., in reverse so that no table is the identity
+    bt = torch.tensor([[1 + t * blocks + (blocks - 1 - b) for b in range(blocks)] for t in range(T)],
+                      dtype=torch.int32, device=DEV)
+    positions = torch.tensor([ctx_len - 1 - 3 * t for t in range(T)], dtype=torch.int32, device=DEV)
+    seq = torch.arange(T, dtype=torch.int32, device=DEV)
+    return q, kp, vp, bt, positions, seq
+
+
+def _both(lib, T, H, G, hd, ps, ctx_len, n_splits, vis, span, seed):
+    from spite_amd.csrc import hipops
+    q, kp, vp, bt, positions, seq = _case(T, H, G, hd, ps, ctx_len, seed)
+    out_ws = torch.zeros(T, H * hd, dtype=torch.bfloat16, device=DEV)
+    out_st = torch.full((T, H * hd), 7.0, dtype=torch.bfloat16, device=DEV)
+    work = torch.empty(hipops.attn_decode_workspace(T, H, hd, n_splits) // 4, dtype=torch.float32, device=DEV)
+    hipops.attn_decode(q, kp, vp, out_ws, work, positions, seq, bt, T, H, G, hd, ps, vis, span, hd ** -0.5, n_splits)
+    torch.cuda.synchronize()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    P = ctypes.c_void_p
+    before = torch.cuda.memory_allocated()
+    rc = lib.spite_attn_decode_static(
+        P(q.data_ptr()), P(kp.data_ptr()), P(vp.data_ptr()), P(out_st.data_ptr()), P(positions.data_ptr()),
+        P(seq.data_ptr()), P(bt.data_ptr()), ctypes.c_int(bt.shape[1]), ctypes.c_int(T), ctypes.c_int(H),
+        ctypes.c_int(G), ctypes.c_int(hd), ctypes.c_int(ps), ctypes.c_int(hipops.VIS[vis]), ctypes.c_int(span),
+        ctypes.c_float(hd ** -0.5), ctypes.c_int(n_splits), stream)
+    assert rc == 0, lib.spite_hip_last_error().decode()
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before
+    assert torch.isfinite(out_st.float()).all()
+    assert torch.equal(out_ws, out_st), (out_ws.float() - out_st.float()).abs().max()
+    return out_st
+
+
+def test_static_scratch_matches_the_workspace_form_twice_in_a_row():
+    from spite_amd.csrc import hipops
+    lib = hipops.lib()
+    lib.spite_attn_decode_static.restype = ctypes.c_int
+    # a larger call first, then a smaller one that finds the first call's records in the array
+    big = _both(lib, T=6, H=40, G=8, hd=128, ps=64, ctx_len=1500, n_splits=16, vis="full", span=0, seed=1)
+    small = _both(lib, T=2, H=8, G=2, hd=64, ps=32, ctx_len=300, n_splits=3, vis="chunk", span=128, seed=2)
+    assert big.shape == (6, 40 * 128) and small.shape == (2, 8 * 64)
+    # one split uses no scratch at all
+    _both(lib, T=3, H=5, G=1, hd=64, ps=32, ctx_len=200, n_splits=1, vis="full", span=0, seed=3)
+
+
+def test_static_scratch_refuses_what_does_not_fit():
+    from spite_amd.csrc import hipops
+    lib = hipops.lib()
+    lib.spite_attn_decode_static.restype = ctypes.c_int
+    T, H, hd, n_splits = 64, 40, 128, 64          # 64*40*64*130 floats, more than the array holds
+    assert T * H * n_splits * (hd + 2) > STATIC_FLOATS
+    z = ctypes.c_void_p(0)
+    rc = lib.spite_attn_decode_static(z, z, z, z, z, z, z, ctypes.c_int(4), ctypes.c_int(T), ctypes.c_int(H),
+                                      ctypes.c_int(8), ctypes.c_int(hd), ctypes.c_int(64), ctypes.c_int(0),
+                                      ctypes.c_int(0), ctypes.c_float(0.1), ctypes.c_int(n_splits), z)
+    assert rc != 0
+    assert "exceed" in lib.spite_hip_last_error().decode()
