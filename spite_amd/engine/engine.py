@@ -124,14 +124,15 @@ class Engine:
                  num_pages=None, cache_tokens: Optional[int] = None, max_batch_tokens: int = 2048,
                  max_requests: int = 8, device: str = "cuda:0", random_weights: bool = False, seed: int = 0,
                  init_std: float = 0.02, spec: Optional[ModelSpec] = None, tensors: Optional[dict] = None,
-                 graphs: bool = True):
+                 graphs: bool = True, workspace_bytes: int = 1 << 20):
         """``model``: a folder with config.json and model.safetensors; with ``random_weights`` a
         folder, a config.json path or a config dict whose weights are drawn on the GPU from
         ``seed``.  ``spec`` (+ ``tensors`` by checkpoint name, or ``random_weights``) builds a
         model from parts directly, without an architecture.  With ``graphs`` a decode step (one
         token of every request, every logit wanted) is captured in a HIP graph the second time
         its shape comes up and replayed from then on: the step is bound by kernel launches
-        otherwise.  The graph holds the same kernels on the same buffers as the eager step."""
+        otherwise.  The graph holds the same kernels on the same buffers as the eager step.
+        ``workspace_bytes``: the first size of the step's scratch buffers, which grow on demand."""
         if dtype not in _DTYPES:
             raise EngineError(f"dtype {dtype!r} (known: bfloat16, float32)")
         if not torch.cuda.is_available():
@@ -170,8 +171,8 @@ class Engine:
             load_weights(self.model, model, ckpt_dtype)
             self._folder = model
         torch.cuda.empty_cache()
-        self._arenas = [Workspace(self.device), Workspace(self.device)]
-        self._step_ws = Workspace(self.device)
+        self._arenas = [Workspace(self.device, workspace_bytes), Workspace(self.device, workspace_bytes)]
+        self._step_ws = Workspace(self.device, workspace_bytes)
         self._pin = None
         self._pin_event = None
         self._meta_dev = None
@@ -314,7 +315,9 @@ class Engine:
                 logits = self.model.forward(meta.ctx, self.cache, meta, self._arenas, self._step_ws)
                 if key is not None:
                     self._graphs[key] = "seen"
-                    self._graph_stamp = self._stamp()
+                # this step may have grown a workspace (a first decode step of a larger shape
+                # does): graphs captured before point into memory that the merge frees
+                self._drop_stale_graphs()
         if commit:
             for e in entries:
                 self.cache.commit(e.slot, len(e.tokens))
@@ -327,10 +330,18 @@ class Engine:
         return (self._meta_dev.data_ptr() if self._meta_dev is not None else 0, self._step_ws.generation,
                 self._arenas[0].generation, self._arenas[1].generation)
 
+    def _drop_stale_graphs(self) -> bool:
+        """Forgets every captured graph if a buffer has moved since the stamp was taken (the
+        marks of shapes seen once are no pointers and stay).  True if something moved."""
+        stamp = self._stamp()
+        if stamp == self._graph_stamp:
+            return False
+        self._graphs = {k: v for k, v in self._graphs.items() if v == "seen"}
+        self._graph_stamp = stamp
+        return True
+
     def _replay(self, key):
-        if self._graph_stamp != self._stamp():
-            self._graphs.clear()           # their addresses are stale
-            self._graph_stamp = self._stamp()
+        if self._drop_stale_graphs():
             return None
         hit = self._graphs.get(key)
         if hit is None or hit == "seen":
@@ -343,6 +354,7 @@ class Engine:
     def _capture(self, key, meta):
         for ws in self._arenas:
             ws.reset()                     # merge what the warm-up step added, outside the capture
+        self._drop_stale_graphs()          # the merge has freed what older graphs point into
         graph = torch.cuda.CUDAGraph()
         try:
             with torch.cuda.graph(graph):
@@ -354,9 +366,12 @@ class Engine:
             warnings.warn("capturing the decode step in a HIP graph failed; steps run eagerly from now on")
             self._step_ws.reset()
             return self.model.forward(meta.ctx, self.cache, meta, self._arenas, self._step_ws)
+        if self._drop_stale_graphs():      # cannot happen (a workspace refuses to grow under capture)
+            self._graphs.pop(key, None)
+            self._step_ws.reset()
+            return self.model.forward(meta.ctx, self.cache, meta, self._arenas, self._step_ws)
         graph.replay()                     # the capture itself computed nothing
         self._graphs[key] = (graph, logits)
-        self._graph_stamp = self._stamp()
         self.graph_replays += 1
         return logits
 

@@ -41,3 +41,47 @@ def test_graph_replays_equal_eager_steps(tmp_path, dtype):
     assert engines[0].graph_replays >= 30 and engines[1].graph_replays == 0
     for a, b in zip(*outs):
         assert a.shape == b.shape and np.array_equal(a, b)
+
+
+def test_a_graph_is_not_replayed_after_a_later_step_has_moved_the_workspaces(tmp_path):
+    # a small decode shape is captured; the first decode step of a larger shape then grows the
+    # scratch buffers (they start tiny here), which frees what the first graph points into; back
+    # at the small shape the graph must be captured anew, not replayed
+    from spite_amd.engine.engine import Engine, StepEntry
+    d = str(tmp_path / "m")
+    H.make_model(d, CFG, seed=4, dtype="bfloat16")
+    prompts = [H.random_tokens(CFG["vocab_size"], 3, 70 + i) for i in range(3)]
+    outs = []
+    for graphs in (True, False):
+        eng = Engine(d, dtype="bfloat16", page_size=32, cache_tokens=1024, max_requests=4, graphs=graphs,
+                     workspace_bytes=2048)
+        rows = []
+        slots = [eng.admit()]
+        tok = [int(eng.step([StepEntry(slots[0], prompts[0], [2])]).argmax(-1)[0])]
+        for _ in range(6):                                   # seen, captured, replayed
+            lg = eng.step([StepEntry(slots[0], [tok[0]], [0])])
+            rows.append(lg.cpu().numpy().copy())
+            tok = lg.argmax(-1).tolist()
+        first = {k: v for k, v in eng._graphs.items() if v != "seen"}
+        assert bool(first) == graphs
+        for p in prompts[1:]:
+            slots.append(eng.admit())
+            tok.append(int(eng.step([StepEntry(slots[-1], p, [2])]).argmax(-1)[0]))
+        before = eng._stamp()
+        for _ in range(3):                                   # three requests: three rows of logits, more scratch
+            lg = eng.step([StepEntry(s, [t], [0]) for s, t in zip(slots, tok)])
+            rows.append(lg.cpu().numpy().copy())
+            tok = lg.argmax(-1).tolist()
+        if graphs:
+            assert eng._stamp() != before, "the larger shape was meant to grow a workspace"
+            assert all(eng._graphs.get(k) is not g for k, g in first.items()), "a stale graph was kept"
+        for s in slots[1:]:
+            eng.release(s)
+        for _ in range(5):                                   # the small shape again
+            lg = eng.step([StepEntry(slots[0], [tok[0]], [0])])
+            rows.append(lg.cpu().numpy().copy())
+            tok = [int(lg.argmax(-1)[0])]
+        outs.append(rows)
+        eng.cache.check()
+    for a, b in zip(*outs):
+        assert a.shape == b.shape and np.array_equal(a, b)
