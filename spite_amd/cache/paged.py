@@ -74,6 +74,7 @@ class PagedCache:
         if not self._h:
             raise CacheError(hostlib.last_error())
         self._lib = lib
+        self._fresh_buf = (ctypes.c_int * (4 * self.max_requests + 4))()
         self.states: Dict[int, torch.Tensor] = {}
         if allocate:
             for g in self.groups:
@@ -104,12 +105,23 @@ class PagedCache:
         slot = self._lib.spc_admit(self._h)
         if slot < 0:
             raise CacheError(f"all {self.max_requests} request slots are taken")
-        self.zero_state(slot)
+        self.zero_fresh()
         return slot
 
-    def zero_state(self, slot: int):
-        for st in self.states.values():
-            st[slot].zero_()
+    def zero_fresh(self) -> List[int]:
+        """Clears the state rows of every slot that has been handed out since the last call, by
+        whomever (this object's ``admit`` or the native scheduler, which admits on its own): the
+        step function calls it before it runs, so a new request never meets the state that the
+        slot's last request left.  Returns those slots."""
+        n = self._lib.spc_take_fresh(self._h, self._fresh_buf, len(self._fresh_buf))
+        if n > len(self._fresh_buf):           # more admissions than slots since the last step: clear them all
+            slots = list(range(self.max_requests))
+        else:
+            slots = sorted(set(self._fresh_buf[:n]))
+        if slots:
+            for st in self.states.values():
+                st[slots] = 0
+        return slots
 
     def live(self, slot):
         return bool(self._lib.spc_live(self._h, slot))
@@ -162,22 +174,21 @@ class PagedCache:
             raise CacheError(hostlib.last_error())
 
     # ------------------------------------------------------------------ step metadata
-    def fill_step(self, slots, starts, counts, g, slot_map_out: np.ndarray, table_out: np.ndarray):
-        """Cache rows of every token of the step and one block-table row per entry."""
-        off = 0
-        width = table_out.shape[1]
-        for i, (s, st, n) in enumerate(zip(slots, starts, counts)):
-            s, st, n = int(s), int(st), int(n)
-            if self._lib.spc_slot_mapping(self._h, s, g, st, n, slot_map_out[off:off + n].ctypes.data) != 0:
-                raise CacheError(f"slot {s} is not live")
-            tl = self._lib.spc_table_len(self._h, s, g)
-            if tl > width:
-                raise CacheError("block table wider than planned")
-            row = table_out[i]
-            row[tl:] = -1
-            if tl:
-                self._lib.spc_table(self._h, s, g, row.ctypes.data_as(ctypes.POINTER(ctypes.c_int)), tl)
-            off += n
+    def fill_step(self, slots: np.ndarray, starts: np.ndarray, counts: np.ndarray, g,
+                  slot_map_out: np.ndarray, table_out: np.ndarray):
+        """Cache rows of every token of the step and one block-table row per entry (int32
+        arrays, contiguous; one native call for the whole step)."""
+        n, width = table_out.shape
+        slots, starts, counts = (np.ascontiguousarray(a, dtype=np.int32) for a in (slots, starts, counts))
+        if not (slot_map_out.dtype == table_out.dtype == np.int32 and slot_map_out.flags.c_contiguous
+                and table_out.flags.c_contiguous and slot_map_out.size >= int(counts.sum()) and len(slots) == n):
+            raise CacheError("fill_step: outputs must be contiguous int32 arrays of the step's sizes")
+        rc = self._lib.spc_fill_step(self._h, n, slots.ctypes.data, starts.ctypes.data, counts.ctypes.data, g, width,
+                                     slot_map_out.ctypes.data, table_out.ctypes.data)
+        if rc == -4:
+            raise CacheError("block table wider than planned")
+        if rc != 0:
+            raise CacheError("a slot of the step is not live")
 
     def table_len(self, slot, g) -> int:
         return int(self._lib.spc_table_len(self._h, slot, g))

@@ -10,6 +10,10 @@ Key map from the reference's GGUF metadata (crates/spite-loader/src/config.rs:22
 ``num_local_experts``; ``expert_used_count`` -> ``num_experts_per_tok``;
 ``interleave_moe_layer_step`` and ``vocab_size`` keep their names.
 
+``attention_local_kind`` (this engine's own key, default ``chunk``) says what a rotating layer
+reads of ``attention_chunk_size`` keys: the chunk its position lies in, or, as the reference's
+forward computes it (crates/spite-models/src/llama/llama4.rs:189-197), a window of the last keys.
+
 What the reference fixes in code is a key here: head size (``d / H`` at
 crates/spite-models/src/llama/llama4.rs:87), the every-fourth-layer rule (:95), qk-norm
 (:96), the temperature constants 8192 and 0.1 (:179).  The reference reads missing keys as
@@ -57,6 +61,7 @@ class Llama4Config:
     rope_scaling: Optional[RopeScaling]
     rope_pairing: str                 # "half" (reference) or "adjacent"
     attention_chunk_size: Optional[int]
+    attention_local_kind: str         # what a rotating layer reads: "chunk" (its chunk) or "window" (the last keys)
     no_rope_layers: Tuple[int, ...]   # 1 = the layer rotates (and is chunked), 0 = NoPE, full causal
     moe_layers: Tuple[int, ...]       # indices of layers with experts
     use_qk_norm: bool
@@ -158,7 +163,8 @@ class Llama4Config:
             rms_norm_eps=opt("rms_norm_eps", float, 1e-5),
             rope_theta=opt("rope_theta", float, 10000.0), rope_scaling=scaling,
             rope_pairing=opt("rope_pairing", str, "half"),
-            attention_chunk_size=chunk, no_rope_layers=nr, moe_layers=moe_layers,
+            attention_chunk_size=chunk, attention_local_kind=opt("attention_local_kind", str, "chunk"),
+            no_rope_layers=nr, moe_layers=moe_layers,
             use_qk_norm=opt("use_qk_norm", bool, True),
             attn_temperature_tuning=opt("attn_temperature_tuning", bool, True),
             floor_scale=opt("floor_scale", int, 8192), attn_scale=opt("attn_scale", float, 0.1),
@@ -198,6 +204,8 @@ class Llama4Config:
                      f"{self.num_hidden_layers} layers")
         if self.rope_pairing not in ("half", "adjacent"):
             p.append(f"rope_pairing {self.rope_pairing!r} (known: 'half', 'adjacent')")
+        if self.attention_local_kind not in ("chunk", "window"):
+            p.append(f"attention_local_kind {self.attention_local_kind!r} (known: 'chunk', 'window')")
         if self.rms_norm_eps <= 0:
             p.append(f"rms_norm_eps must be > 0, got {self.rms_norm_eps}")
         if self.rope_theta <= 0:

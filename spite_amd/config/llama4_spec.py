@@ -13,7 +13,7 @@ from .registry import register_architecture
 from ..parts.base import PartSpec, BlockSpec, LayerCall, ModelSpec
 
 
-def build_spec(cfg: Llama4Config) -> ModelSpec:
+def build_spec(cfg: Llama4Config, ignore_prefixes=()) -> ModelSpec:
     d, H, G, hd = cfg.hidden_size, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
     scaling = None
     if cfg.rope_scaling is not None:
@@ -30,7 +30,7 @@ def build_spec(cfg: Llama4Config) -> ModelSpec:
             position = PartSpec("rotary", {"head_dim": hd, "theta": cfg.rope_theta, "scaling": scaling,
                                            "pairing": cfg.rope_pairing})
             chunked = cfg.attention_chunk_size is not None
-            attn_args = dict(visibility="chunk" if chunked else "full", span=cfg.attention_chunk_size or 0,
+            attn_args = dict(visibility=cfg.attention_local_kind if chunked else "full", span=cfg.attention_chunk_size or 0,
                              qk_norm=cfg.use_qk_norm, qk_norm_eps=cfg.rms_norm_eps, temperature=None)
         else:
             position = PartSpec("none")
@@ -63,7 +63,16 @@ def build_spec(cfg: Llama4Config) -> ModelSpec:
         final_norm=PartSpec("rms", {"width": d, "eps": cfg.rms_norm_eps}, {"weight": "model.norm.weight"}),
         embed_name="model.embed_tokens.weight",
         head_name=None if cfg.tie_word_embeddings else "lm_head.weight",
-        eos_token_ids=cfg.eos_token_ids, max_position=cfg.max_position_embeddings)
+        eos_token_ids=cfg.eos_token_ids, max_position=cfg.max_position_embeddings,
+        ignore_prefixes=tuple(ignore_prefixes))
+
+
+def build_text_spec_of_multimodal(cfg: Llama4Config) -> ModelSpec:
+    """The text model of a checkpoint that also holds a vision tower: its keys lie under
+    ``text_config``, its tensors under ``language_model.``; the other towers' tensors belong to
+    no part of this model and are passed over."""
+    return build_spec(cfg, ignore_prefixes=("vision_model.", "multi_modal_projector."))
 
 
 register_architecture("Llama4ForCausalLM", Llama4Config.from_dict, build_spec)
+register_architecture("Llama4ForConditionalGeneration", Llama4Config.from_dict, build_text_spec_of_multimodal)

@@ -663,27 +663,88 @@ extern "C" int spite_convert(const void* in, int in_dtype, void* out, int out_dt
 // ------------------------------------------------------------------ random weights
 // out[i] = mean + std * z(seed, key, i), z standard normal: element i of a tensor depends on the
 // seed, the tensor's key (a hash of its name) and i alone, not on the order in which tensors
-// or elements are drawn.  A 64-bit mix of (seed, key, i / 2) gives two uniform numbers, and
-// Box-Muller turns them into the normals of the elements i and i + 1.
+// or elements are drawn.  A 64-bit mix of (seed, key, i / 2) gives two uniform numbers of 32 bits,
+// and Box-Muller turns them into the normals of the elements i and i + 1.
+//
+// The same numbers can be drawn on the host, bit for bit: logarithm, sine and cosine are
+// computed here from IEEE double additions, multiplications, divisions and one square root in
+// a fixed order, never fused (a fused multiply-add rounds once where the host rounds twice),
+// instead of the device library's routines, whose last bits differ from a host library's.
 __device__ __forceinline__ unsigned long long mix64(unsigned long long x) {
     x ^= x >> 30; x *= 0xbf58476d1ce4e5b9ull;
     x ^= x >> 27; x *= 0x94d049bb133111ebull;
     return x ^ (x >> 31);
 }
+// ln(x) for x in (0, 1]: x = m * 2^e with m in [sqrt(1/2), sqrt(2)), ln(m) = 2 atanh(s) with
+// s = (m-1)/(m+1), |s| < 0.172: the series up to s^23 is exact to double rounding.
+__device__ __forceinline__ double exact_log(double x) {
+#pragma clang fp contract(off)
+    int e;
+    double m = frexp(x, &e);
+    if (m < 0.70710678118654752) { m = m * 2.0; e -= 1; }
+    const double s = (m - 1.0) / (m + 1.0);
+    const double s2 = s * s;
+    double p = 1.0 / 23.0;
+    p = p * s2 + 1.0 / 21.0;
+    p = p * s2 + 1.0 / 19.0;
+    p = p * s2 + 1.0 / 17.0;
+    p = p * s2 + 1.0 / 15.0;
+    p = p * s2 + 1.0 / 13.0;
+    p = p * s2 + 1.0 / 11.0;
+    p = p * s2 + 1.0 / 9.0;
+    p = p * s2 + 1.0 / 7.0;
+    p = p * s2 + 1.0 / 5.0;
+    p = p * s2 + 1.0 / 3.0;
+    p = p * s2 + 1.0;
+    return (double)e * 0.6931471805599453 + 2.0 * (s * p);
+}
+// sine and cosine of the angle 2 pi k / 2^32: the quadrant from the two top bits, the angle inside
+// it folded to [0, pi/4] (sin(pi/2 - t) = cos t), Taylor sums there up to t^17 and t^18.
+__device__ __forceinline__ void exact_sincos_turns(unsigned k, double& sn, double& cs) {
+#pragma clang fp contract(off)
+    const unsigned quad = k >> 30, low = k & 0x3fffffffu;
+    const bool fold = low > 0x20000000u;
+    const unsigned a = fold ? 0x40000000u - low : low;
+    const double t = (double)a * (1.5707963267948966 / 1073741824.0);
+    const double t2 = t * t;
+    double ps = 1.0 / 355687428096000.0;
+    ps = ps * t2 - 1.0 / 1307674368000.0;
+    ps = ps * t2 + 1.0 / 6227020800.0;
+    ps = ps * t2 - 1.0 / 39916800.0;
+    ps = ps * t2 + 1.0 / 362880.0;
+    ps = ps * t2 - 1.0 / 5040.0;
+    ps = ps * t2 + 1.0 / 120.0;
+    ps = ps * t2 - 1.0 / 6.0;
+    ps = ps * t2 + 1.0;
+    double pc = -1.0 / 6402373705728000.0;
+    pc = pc * t2 + 1.0 / 20922789888000.0;
+    pc = pc * t2 - 1.0 / 87178291200.0;
+    pc = pc * t2 + 1.0 / 479001600.0;
+    pc = pc * t2 - 1.0 / 3628800.0;
+    pc = pc * t2 + 1.0 / 40320.0;
+    pc = pc * t2 - 1.0 / 720.0;
+    pc = pc * t2 + 1.0 / 24.0;
+    pc = pc * t2 - 1.0 / 2.0;
+    pc = pc * t2 + 1.0;
+    const double s0 = fold ? pc : t * ps, c0 = fold ? t * ps : pc;
+    sn = quad == 0 ? s0 : quad == 1 ? c0 : quad == 2 ? -s0 : -c0;
+    cs = quad == 0 ? c0 : quad == 1 ? -s0 : quad == 2 ? -c0 : s0;
+}
 template <typename T>
 __global__ __launch_bounds__(256)
 void randn_fill_kernel(T* __restrict__ out, size_t n, unsigned long long seed, unsigned long long key, float mean, float std) {
+#pragma clang fp contract(off)
     const unsigned long long base = mix64(seed * 0x9e3779b97f4a7c15ull + key);
     const size_t pairs = (n + 1) / 2;
     for (size_t j = (size_t)blockIdx.x * blockDim.x + threadIdx.x; j < pairs; j += (size_t)gridDim.x * blockDim.x) {
         const unsigned long long h = mix64(base + j * 0xd1342543de82ef95ull);
-        const float u1 = ((float)(unsigned)(h >> 40) + 1.0f) * (1.0f / 16777216.0f);          // (0, 1]
-        const float u2 = (float)(unsigned)((h >> 16) & 0xffffff) * (1.0f / 16777216.0f);      // [0, 1)
-        const float r = sqrtf(-2.0f * logf(u1));
-        float sn, cs;
-        sincosf(6.283185307179586f * u2, &sn, &cs);
-        out[2 * j] = from_f32<T>(mean + std * r * cs);
-        if (2 * j + 1 < n) out[2 * j + 1] = from_f32<T>(mean + std * r * sn);
+        const double u1 = ((double)(unsigned)(h >> 32) + 1.0) * (1.0 / 4294967296.0);          // (0, 1]
+        const double r = sqrt(-2.0 * exact_log(u1));
+        double sn, cs;
+        exact_sincos_turns((unsigned)h, sn, cs);
+        const float z0 = (float)(r * cs), z1 = (float)(r * sn);
+        out[2 * j] = from_f32<T>(std * z0 + mean);
+        if (2 * j + 1 < n) out[2 * j + 1] = from_f32<T>(std * z1 + mean);
     }
 }
 extern "C" int spite_randn_fill(void* out, int dtype, size_t n, unsigned long long seed, unsigned long long key,

@@ -109,6 +109,11 @@ def embed(ids, table, h):
                              _ptr(h, "h", torch.float32), T, d, table.shape[0], _stream()), "embed")
 
 
+def add_rmsnorm_can_project(d: int) -> bool:
+    """Whether ``add_rmsnorm`` forms projections of rows of this width (the row stays in LDS)."""
+    return d * 4 <= 48 * 1024
+
+
 def add_rmsnorm(h, w, eps, out=None, out32=None, d1=None, d2=None, rows=None, n_rows=None, write_h=True,
                 proj=None, proj_out=None):
     """v = h[r] + d1[r] + d2[r] (stored back if write_h); out[i] = rmsnorm(v) * w with r =

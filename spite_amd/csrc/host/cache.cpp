@@ -38,7 +38,15 @@ int CacheManager::admit() {
         sl.table[g].clear();
         sl.freed_below[g] = 0;
     }
+    fresh_.push_back(s);
     return s;
+}
+
+int CacheManager::take_fresh(int* out, int cap) {
+    const int n = (int)fresh_.size();
+    for (int i = 0; i < n && i < cap; ++i) out[i] = fresh_[i];
+    fresh_.clear();
+    return n;
 }
 
 bool CacheManager::live(int slot) const {
@@ -140,6 +148,21 @@ void CacheManager::slot_mapping(int slot, int g, int64_t start, int64_t n, int32
         const int page = b < (int64_t)tab.size() ? tab[b] : -1;
         out[i] = page < 0 ? -1 : (int32_t)((int64_t)page * page_size_ + pos % page_size_);
     }
+}
+
+int CacheManager::fill_step(int n, const int32_t* slots, const int32_t* starts, const int32_t* counts, int g,
+                            int width, int32_t* slot_map, int32_t* table) const {
+    int64_t off = 0;
+    for (int i = 0; i < n; ++i) {
+        if (!live(slots[i])) return -2;
+        const auto& tab = slots_[slots[i]].table[g];
+        if ((int)tab.size() > width) return -4;
+        slot_mapping(slots[i], g, starts[i], counts[i], slot_map + off);
+        off += counts[i];
+        int32_t* row = table + (int64_t)i * width;
+        for (int b = 0; b < width; ++b) row[b] = b < (int)tab.size() ? tab[b] : -1;
+    }
+    return 0;
 }
 
 std::string CacheManager::check() const {

@@ -46,6 +46,11 @@ public:
     int free_slots() const { return (int)free_slots_.size(); }
 
     int admit();                               // slot id, or -1 when every slot is taken
+    // Slots handed out since the last call, oldest first (a slot that was admitted, released and
+    // admitted again appears twice): whoever keeps per-request state on the GPU clears the rows
+    // of these slots before the next step runs, whichever caller admitted them.  Returns how
+    // many there were; at most `cap` are written.
+    int take_fresh(int* out, int cap);
     bool live(int slot) const;
     int64_t cached(int slot) const;            // positions committed
     // Pages that reserve(slot, n) would take from group g's pool.
@@ -63,6 +68,11 @@ public:
     const std::vector<int>& table(int slot, int g) const { return slots_[slot].table[g]; }
     // Cache rows (page * page_size + offset) of positions [start, start+n); -1 where no page.
     void slot_mapping(int slot, int g, int64_t start, int64_t n, int32_t* out) const;
+    // For the n entries (slot, first position, count) of a step: the cache rows of all their
+    // tokens in a row in `slot_map`, and one block-table row of `width` entries each in `table`
+    // (-1 past a table's end).  -2: a slot is not live; -4: a table is wider than `width`.
+    int fill_step(int n, const int32_t* slots, const int32_t* starts, const int32_t* counts, int g, int width,
+                  int32_t* slot_map, int32_t* table) const;
     // 0 when every page is either free or in exactly one table, once; else a message.
     std::string check() const;
 
@@ -79,6 +89,7 @@ private:
     std::vector<std::vector<int>> free_;       // [group] stack of free pages
     std::vector<Slot> slots_;
     std::vector<int> free_slots_;              // stack, lowest id on top at the start
+    std::vector<int> fresh_;                   // admitted and not yet reported by take_fresh
 };
 
 }  // namespace spite

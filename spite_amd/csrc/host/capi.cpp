@@ -29,6 +29,11 @@ void* spc_create(int page_size, int max_requests, int n_groups, const int* kinds
 }
 void spc_destroy(void* c) { delete (CacheManager*)c; }
 int spc_admit(void* c) { return ((CacheManager*)c)->admit(); }
+int spc_take_fresh(void* c, int* out, int cap) { return ((CacheManager*)c)->take_fresh(out, cap); }
+int spc_fill_step(void* c, int n, const int* slots, const int* starts, const int* counts, int g, int width,
+                  int* slot_map, int* table) {
+    return ((CacheManager*)c)->fill_step(n, slots, starts, counts, g, width, slot_map, table);
+}
 int spc_live(void* c, int slot) { return ((CacheManager*)c)->live(slot); }
 long long spc_cached(void* c, int slot) { return ((CacheManager*)c)->cached(slot); }
 int spc_can_reserve(void* c, int slot, long long n) { return ((CacheManager*)c)->can_reserve(slot, n); }

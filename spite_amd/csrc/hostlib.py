@@ -21,6 +21,8 @@ def lib():
             "spc_create": (P, [I, I, I, PI, PI, PI]),
             "spc_destroy": (None, [P]),
             "spc_admit": (I, [P]),
+            "spc_take_fresh": (I, [P, PI, I]),
+            "spc_fill_step": (I, [P, I, c_void_p, c_void_p, c_void_p, I, I, c_void_p, c_void_p]),
             "spc_live": (I, [P, I]),
             "spc_cached": (LL, [P, I]),
             "spc_can_reserve": (I, [P, I, LL]),

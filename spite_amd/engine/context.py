@@ -96,6 +96,5 @@ class StepContext:
     ws: Any = None               # Workspace of the layer call that runs
     decode_only: bool = False    # every entry holds one token
     max_count: int = 0           # longest portion of the step
-    lead_singles: int = 0        # in a mixed step: how many entries of one token each come first
-    cu_tail: Optional[torch.Tensor] = None   # int32: cu_seqlens of the entries behind them, from 0
+    derived: dict = field(default_factory=dict)   # step arrays that parts asked for: name -> (device array, info)
     extras: dict = field(default_factory=dict)

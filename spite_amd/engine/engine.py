@@ -18,8 +18,8 @@ import torch
 from ..cache.paged import PagedCache
 from ..config import read_config
 from ..csrc import hipops
-from ..parts.base import ModelSpec, LayerCall
-from ..weights.loader import load_weights
+from ..parts.base import ModelSpec, LayerCall, step_array_builder
+from ..weights.loader import bind, FolderSource, DictSource, RandomSource
 from .context import Env, Workspace, StepContext, LayerCache, HostBatch
 from .model import Model
 
@@ -65,16 +65,13 @@ class StepMeta:
                     raise EngineError(f"entry {i}: wanted place {w} outside its {counts[i]} tokens")
                 rows.append(int(cu[i]) + int(w))
         n_out = len(rows)
-        # single decoded tokens that lead a mixed step (the scheduler's order): the mixer may give
-        # them to its decode kernel and only the portions behind them to the prefill kernel
-        lead = 0
-        while lead < n and counts[lead] == 1:
-            lead += 1
-        if lead == n:
-            lead = 0
+        # arrays that parts of this model derive from the batch (declared in ``step_arrays``)
+        hb = HostBatch(slots=slots, starts=starts, counts=counts, cu_seqlens=cu)
+        derived = {name: step_array_builder(name)(hb) for name in engine.model.step_arrays}
         # layout of the one int32 buffer
         sizes = [("token_ids", T), ("positions", T), ("seq_of_token", T), ("cu_seqlens", n + 1),
-                 ("seq_slots", n), ("seq_starts", n), ("logit_rows", n_out), ("cu_tail", n - lead + 1 if lead else 0)]
+                 ("seq_slots", n), ("seq_starts", n), ("logit_rows", n_out)]
+        sizes += [(f"derived:{name}", int(arr.size)) for name, (arr, _) in derived.items()]
         for g in range(n_groups):
             sizes += [(f"slot_map{g}", T), (f"table{g}", n * widths[g])]
         offs, total = {}, 0
@@ -86,11 +83,12 @@ class StepMeta:
         tok = hv["token_ids"]
         for i, e in enumerate(entries):
             tok[cu[i]:cu[i + 1]] = np.asarray(e.tokens, dtype=np.int64)
-            hv["positions"][cu[i]:cu[i + 1]] = np.arange(starts[i], starts[i] + counts[i], dtype=np.int32)
-            hv["seq_of_token"][cu[i]:cu[i + 1]] = i
+        # position of token j of entry i: starts[i] + j
+        hv["positions"][:] = np.arange(T, dtype=np.int32) + np.repeat(starts - cu[:-1], counts)
+        hv["seq_of_token"][:] = np.repeat(np.arange(n, dtype=np.int32), counts)
         hv["cu_seqlens"][:] = cu
-        if lead:
-            hv["cu_tail"][:] = cu[lead:] - cu[lead]
+        for name, (arr, _) in derived.items():
+            hv[f"derived:{name}"][:] = arr
         hv["seq_slots"][:] = slots
         hv["seq_starts"][:] = starts
         hv["logit_rows"][:] = np.asarray(rows, dtype=np.int32)
@@ -104,9 +102,8 @@ class StepMeta:
             T=T, n_seqs=n, token_ids=dv["token_ids"], positions=dv["positions"], seq_of_token=dv["seq_of_token"],
             cu_seqlens=dv["cu_seqlens"], seq_slots=dv["seq_slots"], seq_starts=dv["seq_starts"],
             logit_rows=dv["logit_rows"], n_out=n_out,
-            host=HostBatch(slots=slots, starts=starts, counts=counts, cu_seqlens=cu),
-            decode_only=bool(n > 0 and counts.max() == 1), max_count=int(counts.max()) if n else 0,
-            lead_singles=lead, cu_tail=dv["cu_tail"] if lead else None)
+            host=hb, decode_only=bool(n > 0 and counts.max() == 1), max_count=int(counts.max()) if n else 0,
+            derived={name: (dv[f"derived:{name}"], info) for name, (_, info) in derived.items()})
         self.host_tokens = tok[:T].copy()
 
     def layer_cache(self, cache: PagedCache, call: LayerCall) -> LayerCache:
@@ -142,7 +139,7 @@ class Engine:
         torch.cuda.set_device(self.device)
         self.env = Env(_DTYPES[dtype], self.device)
         self.config = None
-        ckpt_dtype = torch.bfloat16
+        ckpt_dtype = self.env.dtype
         if spec is None:
             if model is None:
                 raise EngineError("Engine needs a model folder, a configuration or a spec")
@@ -160,16 +157,15 @@ class Engine:
             tokens = cache_tokens if cache_tokens is not None else self.max_requests * 4096
             num_pages = max(1, -(-int(tokens) // self.page_size))
         self.cache = PagedCache(needs, self.page_size, num_pages, self.max_requests, self.env.dtype, self.device)
-        self._folder = None
         if tensors is not None:
-            self._load_from_dict(tensors, ckpt_dtype)
+            self._source = DictSource(tensors)
         elif random_weights:
-            self._init_random(seed, init_std)
+            self._source = RandomSource(self.model.tensor_plan(), seed, init_std, ckpt_dtype)
         else:
             if not isinstance(model, str) or not os.path.isdir(model):
                 raise EngineError("without random_weights the model must be a folder with model.safetensors")
-            load_weights(self.model, model, ckpt_dtype)
-            self._folder = model
+            self._source = FolderSource(model, spec.strip_prefixes, spec.ignore_prefixes)
+        bind(self.model, self._source, ckpt_dtype)
         torch.cuda.empty_cache()
         self._arenas = [Workspace(self.device, workspace_bytes), Workspace(self.device, workspace_bytes)]
         self._step_ws = Workspace(self.device, workspace_bytes)
@@ -183,65 +179,18 @@ class Engine:
         self.graph_replays = 0
 
     # ------------------------------------------------------------------ weights
-    def _load_from_dict(self, tensors: Dict[str, torch.Tensor], ckpt_dtype):
-        from ..weights.loader import resident_dtype, WeightsError
-        plan = self.model.tensor_plan()
-        names = {f for f, _, _, _ in plan}
-        missing = sorted(n for n in names if n not in tensors)
-        unexpected = sorted(n for n in tensors if n not in names)
-        shapes = [(f, tuple(tensors[f].shape), ps.shape) for f, ps, _, _ in plan
-                  if f in tensors and tuple(tensors[f].shape) != tuple(ps.shape)]
-        if missing or unexpected or shapes:
-            raise WeightsError(missing, unexpected, shapes, (), "the given tensors")
-        by_owner = {}
-        for f, ps, owner, local in plan:
-            t = tensors[f]
-            by_owner.setdefault(id(owner), (owner, {}))[1][local] = t.to(
-                device=self.device, dtype=resident_dtype(t.dtype, ps.kind, self.env.dtype, ckpt_dtype))
-        for owner, ts in by_owner.values():
-            owner.load(ts)
-        self.model.finish_loading()
-
-    def _init_random(self, seed: int, std: float):
-        """Draws every tensor on the GPU in its resident dtype: N(0,std), norm weights 1+N(0,std).
-        The numbers of a tensor depend on the seed, the tensor's name and the element's index
-        alone (``hipops.randn_fill``)."""
-        import zlib
-        by_owner = {}
-        for f, ps, owner, local in self.model.tensor_plan():
-            if ps.kind == "int":
-                t = torch.zeros(ps.shape, dtype=torch.int32, device=self.device)
-            else:
-                dt = torch.float32 if ps.kind == "vector" else self.env.dtype
-                t = torch.empty(ps.shape, dtype=dt, device=self.device)
-                if ps.init == "zeros":
-                    t.zero_()
-                else:
-                    hipops.randn_fill(t, seed, zlib.crc32(f.encode()), 1.0 if ps.init == "ones" else 0.0, std)
-            by_owner.setdefault(id(owner), (owner, {}))[1][local] = t
-        for owner, ts in by_owner.values():
-            owner.load(ts)
-            ts.clear()
-        self.model.finish_loading()
-
     def tensor_names(self):
         """Checkpoint names of the model's tensors, in the order of the layers."""
         return [f for f, _, _, _ in self.model.tensor_plan()]
 
     def get_tensor(self, name: str) -> torch.Tensor:
-        """A tensor of the model folder by its checkpoint name, as stored (on the host).  The
-        parts keep their own layouts of it on the GPU (fused, transposed, in operand order);
-        this reads the file."""
-        if self._folder is None:
-            raise EngineError("get_tensor reads the model folder; this engine was built from tensors in memory "
-                              "(write a folder with `spite random-model` to read them back)")
-        from ..weights.safetensors_io import Checkpoint
-        from ..weights.loader import _strip
-        ckpt = Checkpoint(self._folder)
-        for stored in ckpt.names():
-            if _strip(stored) == name or stored == name:
-                return ckpt.tensor(stored)
-        raise KeyError(f"{name!r} is not a tensor of {self._folder}")
+        """A tensor of the model by its checkpoint name, as its source stores it, on the host:
+        read from the model folder, taken from the tensors given in memory, or drawn again from
+        the seed (the same numbers as the GPU drew).  The parts keep their own layouts of it on
+        the GPU (fused, transposed, in operand order)."""
+        if name not in self._source.names():
+            raise KeyError(f"{name!r} is not a tensor of {self._source.where}")
+        return self._source.host(name)
 
     # ------------------------------------------------------------------ metadata transport
     def _pinned(self, n: int) -> np.ndarray:
@@ -296,6 +245,7 @@ class Engine:
                 bad = int(toks[(toks < 0) | (toks >= V)][0])
                 raise EngineError(f"entry {i}: token id {bad} outside the vocabulary of {V}")
             total += len(e.tokens)
+        self.cache.zero_fresh()       # state rows of slots handed out since the last step, by whomever
         for e in entries:
             self.cache.reserve(e.slot, len(e.tokens))
         meta = StepMeta(self, entries)

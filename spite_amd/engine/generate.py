@@ -51,11 +51,7 @@ def generate(engine, prompts: Sequence[Sequence[int]], max_tokens: int = 16, tem
             if not outs:
                 raise RuntimeError("scheduler made no progress")
         else:
-            entries = []
-            for b in batch:
-                if b.start == 0:
-                    engine.cache.zero_state(b.slot)
-                entries.append(StepEntry(b.slot, b.tokens, [len(b.tokens) - 1] if b.wants_logits else []))
+            entries = [StepEntry(b.slot, b.tokens, [len(b.tokens) - 1] if b.wants_logits else []) for b in batch]
             logits = engine.step(entries, commit=False)
             wanted = [b.request_id for b in batch if b.wants_logits]
             states = [rng[r] for r in wanted]

@@ -34,6 +34,7 @@ class Model:
                 raise ValueError(f"layer call {i} reads cache {call.cache} before any call has written it")
         self._writers = writers
         self.graph_safe = all(b.graph_safe for b in self.blocks) and self.final_norm.graph_safe
+        self.step_arrays = tuple(sorted({a for b in self.blocks for a in b.step_arrays}))
 
     # ------------------------------------------------------------------ tensors
     def tensor_plan(self) -> List[Tuple[str, ParamSpec, object, str]]:

@@ -12,16 +12,37 @@ from __future__ import annotations
 
 import math
 
+import numpy as np
 import torch
 
-from .base import Mixer, ParamSpec, CacheNeed, KVNeed, register, build as build_part
+from .base import Mixer, ParamSpec, CacheNeed, KVNeed, register, register_step_array, build as build_part
 from .linear import linear, Weight
 from ..csrc import hipops
+
+
+def _tail_after_singles(host):
+    """For a mixed step whose first entries hold one token each (decoded tokens lead, the
+    scheduler's order): how many they are, and the running token counts of the entries behind
+    them, from zero.  The decode kernel then takes the singles and the prefill kernel the rest;
+    a query alone would fill a 256-column tile of the prefill kernel with a few columns."""
+    counts, cu = host.counts, host.cu_seqlens
+    n = len(counts)
+    lead = 0
+    while lead < n and counts[lead] == 1:
+        lead += 1
+    if lead == n or lead == 0:
+        return np.zeros(0, dtype=np.int32), 0
+    return (cu[lead:] - cu[lead]).astype(np.int32), lead
+
+
+TAIL = "attention.tail_after_singles"
+register_step_array(TAIL, _tail_after_singles)
 
 
 @register("mixer", "attention")
 class Attention(Mixer):
     graph_safe = True
+    step_arrays = (TAIL,)
 
     def __init__(self, env, hidden_size, n_heads, n_kv_heads, head_dim, position, visibility="full", span=0,
                  qk_norm=False, qk_norm_eps=1e-5, temperature=None, softmax_scale=None):
@@ -100,12 +121,11 @@ class Attention(Mixer):
         if ctx.decode_only and mfma and H // G <= 16:
             self._decode(q, o, ctx, cache, T)
         elif mfma:
-            lead = ctx.lead_singles if H // G <= 16 else 0
-            if lead:
-                # decoded tokens of other requests beside prompt portions: a query alone would
-                # fill a 256-column tile of the prefill kernel with five columns
+            cu_tail, lead = ctx.derived[TAIL]
+            if lead and H // G <= 16:
+                # decoded tokens of other requests beside prompt portions
                 self._decode(q, o, ctx, cache, lead)
-                hipops.attn_prefill(q[lead:], cache.k_pages, cache.v_pages, o[lead:], ctx.positions[lead:], ctx.cu_tail,
+                hipops.attn_prefill(q[lead:], cache.k_pages, cache.v_pages, o[lead:], ctx.positions[lead:], cu_tail,
                                     ctx.host.counts[lead:], cache.block_table[lead:], H, G, hd, cache.page_size,
                                     self.visibility, self.span, self.scale)
             else:

@@ -82,6 +82,8 @@ class ModelSpec:
     head_name: Optional[str]     # None: the embedding table is the output matrix
     eos_token_ids: Tuple[int, ...] = ()
     max_position: int = 1 << 20  # the default context limit of generation (the step function itself has none)
+    strip_prefixes: Tuple[str, ...] = ("language_model.",)   # taken off the checkpoint's tensor names
+    ignore_prefixes: Tuple[str, ...] = ()   # tensors of the checkpoint that belong to no part of this model
 
 
 class Part:
@@ -92,6 +94,10 @@ class Part:
     #: reads the step's metadata on the host (``ctx.host``) must leave this False.
     graph_safe = False
 
+    #: names of derived arrays of the step's metadata that ``forward`` reads from
+    #: ``ctx.derived`` (see ``register_step_array``)
+    step_arrays: Tuple[str, ...] = ()
+
     def params(self) -> Dict[str, ParamSpec]:
         return {}
 
@@ -100,9 +106,11 @@ class Part:
 
 
 class Norm(Part):
-    #: True when forward() takes ``proj`` / ``proj_out``: a small fp32 matrix [P, d] whose
-    #: products with the normed fp32 rows are formed in the same pass (router logits)
-    projects = False
+    def can_project(self, proj) -> bool:
+        """Whether forward() takes this ``proj`` with a ``proj_out``: a small fp32 matrix [P, d]
+        whose products with the normed fp32 rows are formed in the same pass (router logits).
+        The norm knows what its kernel can hold."""
+        return False
 
     def forward(self, h, out, *, d1=None, d2=None, out32=None, rows=None, write_h=True) -> None:
         """h (fp32 [T,d]) += d1 + d2 (kept if write_h); out[i] (and out32[i]) = norm(h[r]), r =
@@ -153,6 +161,26 @@ class Block(Part):
         """Runs the layer on the residual stream h (fp32 [T,d]); ``pending`` are up to two
         increments not yet added to h.  Returns the new pending increments."""
         raise NotImplementedError
+
+
+# ----------------------------------------------------------------------------- derived step metadata
+_STEP_ARRAYS: Dict[str, Callable] = {}
+
+
+def register_step_array(name: str, fn: Callable) -> None:
+    """``fn(host) -> (int32 numpy array, info)``: an array derived from the step's metadata on
+    the host (``host``: slots, starts, counts, cu_seqlens of the entries) that a part's kernels
+    want on the GPU.  It is computed only for models in which a part lists ``name`` in its
+    ``step_arrays``, travels in the step's one metadata copy, and is found under
+    ``ctx.derived[name]`` as ``(device array, info)``; ``info`` is any host-side fact that goes
+    with it.  The function must depend on its argument alone."""
+    _STEP_ARRAYS[name] = fn
+
+
+def step_array_builder(name: str) -> Callable:
+    if name not in _STEP_ARRAYS:
+        raise KeyError(f"no step array {name!r} is registered (known: {sorted(_STEP_ARRAYS)})")
+    return _STEP_ARRAYS[name]
 
 
 # ----------------------------------------------------------------------------- registries

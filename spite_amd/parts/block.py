@@ -22,6 +22,7 @@ class PreNormBlock(Block):
         self.children = (("norm1", self.norm1, spec.norm1), ("mixer", self.mixer, spec.mixer),
                          ("norm2", self.norm2, spec.norm2), ("ffn", self.ffn, spec.ffn))
         self.graph_safe = all(part.graph_safe for _, part, _ in self.children)
+        self.step_arrays = tuple(sorted({a for _, part, _ in self.children for a in part.step_arrays}))
 
     def forward(self, h, pending, ctx, cache):
         T, d = h.shape
@@ -32,8 +33,8 @@ class PreNormBlock(Block):
         self.norm1.forward(h, n, d1=d1, d2=d2)
         delta = self.mixer.forward(n, ctx, cache)
         n2 = ws.take((T, d), self.env.dtype)
-        proj = self.ffn.input_projection() if self.norm2.projects else None
-        if proj is not None and proj.shape[1] * 4 <= 48 * 1024:
+        proj = self.ffn.input_projection()
+        if proj is not None and self.norm2.can_project(proj):
             # the norm forms the feed-forward's small fp32 products (router logits) itself
             logits = ws.take((T, proj.shape[0]), torch.float32)
             self.norm2.forward(h, n2, d1=delta, proj=proj, proj_out=logits)

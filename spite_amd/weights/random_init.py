@@ -1,8 +1,9 @@
 """Random-weights mode: writes a model folder (config.json, model.safetensors) from a
 configuration and a seed.
 
-Every tensor is drawn from its own generator, seeded by (seed, crc32 of the tensor's name),
-so the numbers do not depend on the order of the tensors.  Matrices are N(0, std); norm
+Element i of a tensor is a function of (seed, crc32 of the tensor's name, i) alone, so the
+numbers do not depend on the order of drawing, and the engine's own random-weights mode, which
+draws on the GPU, holds the model that the folder of the same seed holds.  Matrices are N(0, std); norm
 weights 1 + N(0, std) (weights near zero would scale every activation down to where
 attention is uniform and every logit near a tie).  The choice is recorded in config.json
 under ``spite_random_init``.
@@ -14,6 +15,7 @@ import os
 import zlib
 from typing import Dict
 
+import numpy as np
 import torch
 
 from ..config import read_config
@@ -23,15 +25,113 @@ from .safetensors_io import write_safetensors
 _FILE_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "float16": torch.float16}
 
 
+_M64 = (1 << 64) - 1
+
+
+def _mix64(x: np.ndarray) -> np.ndarray:
+    x = x ^ (x >> np.uint64(30))
+    x = x * np.uint64(0xbf58476d1ce4e5b9)
+    x = x ^ (x >> np.uint64(27))
+    x = x * np.uint64(0x94d049bb133111eb)
+    return x ^ (x >> np.uint64(31))
+
+
+def _exact_log(x: np.ndarray) -> np.ndarray:
+    m, e = np.frexp(x)
+    small = m < 0.70710678118654752
+    m = np.where(small, m * 2.0, m)
+    e = np.where(small, e - 1, e)
+    s = (m - 1.0) / (m + 1.0)
+    s2 = s * s
+    p = np.full_like(s, 1.0 / 23.0)
+    for k in (21.0, 19.0, 17.0, 15.0, 13.0, 11.0, 9.0, 7.0, 5.0, 3.0):
+        p = p * s2 + 1.0 / k
+    p = p * s2 + 1.0
+    return e.astype(np.float64) * 0.6931471805599453 + 2.0 * (s * p)
+
+
+def _exact_sincos_turns(k: np.ndarray):
+    quad = k >> np.uint32(30)
+    low = k & np.uint32(0x3fffffff)
+    fold = low > np.uint32(0x20000000)
+    a = np.where(fold, np.uint32(0x40000000) - low, low)
+    t = a.astype(np.float64) * (1.5707963267948966 / 1073741824.0)
+    t2 = t * t
+    ps = np.full_like(t, 1.0 / 355687428096000.0)
+    for sign, f in ((-1, 1307674368000.0), (1, 6227020800.0), (-1, 39916800.0), (1, 362880.0), (-1, 5040.0),
+                    (1, 120.0), (-1, 6.0)):
+        ps = ps * t2 + 1.0 / f if sign > 0 else ps * t2 - 1.0 / f
+    ps = ps * t2 + 1.0
+    pc = np.full_like(t, -1.0 / 6402373705728000.0)
+    for sign, f in ((1, 20922789888000.0), (-1, 87178291200.0), (1, 479001600.0), (-1, 3628800.0), (1, 40320.0),
+                    (-1, 720.0), (1, 24.0), (-1, 2.0)):
+        pc = pc * t2 + 1.0 / f if sign > 0 else pc * t2 - 1.0 / f
+    pc = pc * t2 + 1.0
+    tps = t * ps
+    s0 = np.where(fold, pc, tps)
+    c0 = np.where(fold, tps, pc)
+    sn = np.select([quad == 0, quad == 1, quad == 2], [s0, c0, -s0], -c0)
+    cs = np.select([quad == 0, quad == 1, quad == 2], [c0, -s0, -c0], s0)
+    return sn, cs
+
+
+def normal_numbers(n: int, seed: int, key: int, mean: float = 0.0, std: float = 1.0) -> np.ndarray:
+    """float32 [n]: the numbers that the kernel ``randn_fill`` writes for (seed, key), bit for bit.
+    Element i depends on (seed, key, i) alone.  A 64-bit mix of (seed, key, i // 2) gives two
+    uniform numbers of 32 bits; Box-Muller turns them into the normals of elements i and i + 1;
+    logarithm, sine and cosine are sums of IEEE double operations in a fixed order (the kernel
+    forms the same sums without fused multiply-adds), so both sides round alike."""
+    base = (int(seed) * 0x9e3779b97f4a7c15 + int(key)) & _M64
+    out = np.empty(n, dtype=np.float32)
+    pairs = (n + 1) // 2
+    step = 1 << 20
+    with np.errstate(over="ignore"):
+        base = _mix64(np.array([base], dtype=np.uint64))[0]
+        for j0 in range(0, pairs, step):
+            j = np.arange(j0, min(j0 + step, pairs), dtype=np.uint64)
+            h = _mix64(base + j * np.uint64(0xd1342543de82ef95))
+            u1 = ((h >> np.uint64(32)).astype(np.float64) + 1.0) * (1.0 / 4294967296.0)
+            r = np.sqrt(-2.0 * _exact_log(u1))
+            sn, cs = _exact_sincos_turns((h & np.uint64(0xffffffff)).astype(np.uint32))
+            z0 = (r * cs).astype(np.float32)
+            z1 = (r * sn).astype(np.float32)
+            both = np.empty(2 * len(j), dtype=np.float32)
+            both[0::2] = np.float32(std) * z0 + np.float32(mean)
+            both[1::2] = np.float32(std) * z1 + np.float32(mean)
+            out[2 * j0:2 * j0 + min(2 * len(j), n - 2 * j0)] = both[:n - 2 * j0]
+    return out
+
+
+def tensor_key(name: str) -> int:
+    return zlib.crc32(name.encode())
+
+
 def draw(name: str, spec, seed: int, std: float) -> torch.Tensor:
-    g = torch.Generator(device="cpu")
-    g.manual_seed((int(seed) * 1000003 + zlib.crc32(name.encode())) % (1 << 63))
+    """The tensor ``name`` of a random model, on the host, fp32 (int32 tables are zero)."""
     if spec.kind == "int":
         return torch.zeros(spec.shape, dtype=torch.int32)
     if spec.init == "zeros":
         return torch.zeros(spec.shape, dtype=torch.float32)
-    t = torch.randn(spec.shape, generator=g, dtype=torch.float32) * std
-    return t + 1.0 if spec.init == "ones" else t
+    n = 1
+    for s in spec.shape:
+        n *= int(s)
+    z = normal_numbers(n, seed, tensor_key(name), 1.0 if spec.init == "ones" else 0.0, std)
+    return torch.from_numpy(z).view(tuple(spec.shape))
+
+
+def draw_on_device(name: str, spec, seed: int, std: float, file_dtype: torch.dtype, device) -> torch.Tensor:
+    """The same tensor drawn by the kernel on the GPU, rounded to ``file_dtype`` as the folder
+    of that seed stores it."""
+    from ..csrc import hipops
+    if spec.kind == "int":
+        return torch.zeros(spec.shape, dtype=torch.int32, device=device)
+    direct = file_dtype in (torch.float32, torch.bfloat16)
+    t = torch.empty(spec.shape, dtype=file_dtype if direct else torch.float32, device=device)
+    if spec.init == "zeros":
+        t.zero_()
+    else:
+        hipops.randn_fill(t, seed, tensor_key(name), 1.0 if spec.init == "ones" else 0.0, std)
+    return t if direct else t.to(file_dtype)
 
 
 def random_tensors(config: dict, seed: int, std: float = 0.02) -> Dict[str, torch.Tensor]:

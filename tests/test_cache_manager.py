@@ -174,3 +174,28 @@ def test_random_orders_of_requests_keep_the_books(seed):
     for s in list(live):
         c.release(s)
     assert all(c.free_pages(g) == c.total_pages(g) for g in range(3))
+
+
+def test_slots_handed_out_are_reported_once_whoever_admitted_them():
+    # the native scheduler admits behind the Python object's back; the state rows of every slot
+    # handed out are cleared before the next step, so a request never meets its predecessor's state
+    from spite_amd.engine.scheduler import Scheduler
+    need = CacheNeed(kv=KVNeed(1, 16, "full"), state=StateNeed((3,), torch.float32))
+    c = PagedCache([need], 16, 8, 3, torch.float32, torch.device("cpu"))
+    c.states[0][:] = 7.0
+    s = c.admit()
+    assert c.states[0][s].abs().sum() == 0 and c.states[0].abs().sum() == 2 * 3 * 7.0
+    assert c.zero_fresh() == []
+    c.states[0][:] = 7.0
+    sched = Scheduler(c, 32, 1000)
+    sched.submit([1, 2, 3], 4)
+    sched.submit([4, 5], 4)
+    batch = sched.schedule()                                # admits two slots natively
+    assert sorted(b.slot for b in batch) == [1, 2]
+    assert c.states[0][1:].abs().sum() > 0                  # nothing cleared yet
+    assert c.zero_fresh() == [1, 2]
+    assert c.states[0][1:].abs().sum() == 0 and c.states[0][s].abs().sum() == 21.0
+    assert c.zero_fresh() == []
+    # released and admitted again between two steps: reported, once
+    c.release(s)
+    assert c.admit() == s and c.states[0][s].abs().sum() == 0

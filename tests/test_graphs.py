@@ -50,14 +50,14 @@ def test_a_graph_is_not_replayed_after_a_later_step_has_moved_the_workspaces(tmp
     from spite_amd.engine.engine import Engine, StepEntry
     d = str(tmp_path / "m")
     H.make_model(d, CFG, seed=4, dtype="bfloat16")
-    prompts = [H.random_tokens(CFG["vocab_size"], 3, 70 + i) for i in range(3)]
+    prompts = [H.random_tokens(CFG["vocab_size"], 1 if i == 0 else 2, 70 + i) for i in range(7)]
     outs = []
     for graphs in (True, False):
-        eng = Engine(d, dtype="bfloat16", page_size=32, cache_tokens=1024, max_requests=4, graphs=graphs,
-                     workspace_bytes=2048)
+        eng = Engine(d, dtype="bfloat16", page_size=32, cache_tokens=1024, max_requests=8, graphs=graphs,
+                     workspace_bytes=1024)
         rows = []
         slots = [eng.admit()]
-        tok = [int(eng.step([StepEntry(slots[0], prompts[0], [2])]).argmax(-1)[0])]
+        tok = [int(eng.step([StepEntry(slots[0], prompts[0], [0])]).argmax(-1)[0])]
         for _ in range(6):                                   # seen, captured, replayed
             lg = eng.step([StepEntry(slots[0], [tok[0]], [0])])
             rows.append(lg.cpu().numpy().copy())
@@ -66,9 +66,9 @@ def test_a_graph_is_not_replayed_after_a_later_step_has_moved_the_workspaces(tmp
         assert bool(first) == graphs
         for p in prompts[1:]:
             slots.append(eng.admit())
-            tok.append(int(eng.step([StepEntry(slots[-1], p, [2])]).argmax(-1)[0]))
+            tok.append(int(eng.step([StepEntry(slots[-1], p, [1])]).argmax(-1)[0]))
         before = eng._stamp()
-        for _ in range(3):                                   # three requests: three rows of logits, more scratch
+        for _ in range(3):                                   # seven requests: seven rows of logits, more scratch
             lg = eng.step([StepEntry(s, [t], [0]) for s, t in zip(slots, tok)])
             rows.append(lg.cpu().numpy().copy())
             tok = lg.argmax(-1).tolist()

@@ -724,3 +724,18 @@ def test_randn_fill_is_normal_and_depends_on_seed_key_and_index_alone():
     h = torch.empty(1001, dtype=torch.bfloat16, device=DEV)
     ops().randn_fill(h, 7, 99, 0.0, 1.0)
     assert torch.equal(h, a[:1001].to(torch.bfloat16))
+
+
+def test_randn_fill_equals_its_host_port_bit_for_bit():
+    # the folder writer draws on the host what the engine's random-weights mode draws on the GPU
+    import numpy as np
+    from spite_amd.weights.random_init import normal_numbers
+    n = (1 << 20) + 1
+    for seed, key, mean, std in ((7, 99, 0.0, 1.0), (123456789012345, 0xfedcba98, 1.0, 0.02), (0, 0, 0.0, 0.05)):
+        host = normal_numbers(n, seed, key, mean, std)
+        a = torch.empty(n, device=DEV)
+        ops().randn_fill(a, seed, key, mean, std)
+        assert np.array_equal(a.cpu().numpy().view(np.uint32), host.view(np.uint32)), (seed, key)
+        h = torch.empty(n, dtype=torch.bfloat16, device=DEV)
+        ops().randn_fill(h, seed, key, mean, std)
+        assert torch.equal(h.cpu(), torch.from_numpy(host).to(torch.bfloat16))

@@ -48,7 +48,7 @@ def define_parts():
             return out
 
 
-def spec():
+def spec(vis="window", span=6):
     from spite_amd.parts import PartSpec, BlockSpec, LayerCall, ModelSpec
     norm = lambda name: PartSpec("rms", {"width": D, "eps": 1e-5}, {"weight": name})
     ffn = lambda p: PartSpec("dense_glu", {"hidden_size": D, "intermediate_size": 48},
@@ -59,8 +59,8 @@ def spec():
         {k: f"{p}.{k}" for k in ("q_proj", "k_proj", "v_proj", "o_proj")})
     blocks = [
         BlockSpec("prenorm", norm("b0.n1"), PartSpec("toy_running_mean", {"width": D}, {"proj": "b0.mix"}), norm("b0.n2"), ffn("b0.ffn")),
-        BlockSpec("prenorm", norm("b1.n1"), attn("b1.attn", "window", 6), norm("b1.n2"), ffn("b1.ffn")),
-        BlockSpec("prenorm", norm("b2.n1"), attn("b2.attn", "window", 6), norm("b2.n2"), ffn("b2.ffn")),
+        BlockSpec("prenorm", norm("b1.n1"), attn("b1.attn", vis, span), norm("b1.n2"), ffn("b1.ffn")),
+        BlockSpec("prenorm", norm("b2.n1"), attn("b2.attn", vis, span), norm("b2.n2"), ffn("b2.ffn")),
     ]
     order = [LayerCall(0, 0), LayerCall(1, 1), LayerCall(0, 2), LayerCall(1, 3),      # blocks 0 and 1 run twice
              LayerCall(2, 1, write=False)]                                             # block 2 reads cache 1
@@ -81,7 +81,7 @@ def tensors(seed=0):
     return t
 
 
-def plain_toy(t, tokens):
+def plain_toy(t, tokens, vis="window", span=6):
     """The same model, whole sequence, in float64 torch."""
     import plain_llama4 as plain
     W = {k: v.double() for k, v in t.items()}
@@ -89,7 +89,7 @@ def plain_toy(t, tokens):
     pos = torch.arange(T)
     h = W["embed"][torch.tensor(tokens)]
     inv = plain.rope_inv_freq(HD, 100.0, None)
-    mask = plain.visible_mask(pos, "window", 6)
+    mask = plain.visible_mask(pos, vis, span)
     kv = {}
 
     def ffn(b, x):
@@ -155,3 +155,30 @@ def test_an_unknown_part_or_a_bad_order_is_refused():
     sp.order.append(LayerCall(1, 1))
     with pytest.raises(ValueError, match="written by layer calls"):
         Engine(spec=sp, tensors=tensors(), dtype="float32")
+
+
+def test_the_toy_mixer_is_served_by_generate_with_preemption_on_a_tiny_pool():
+    # requests come and go through the native scheduler, which hands out slots on its own and
+    # preempts when the pages run out: a request that gets a used slot, or is recomputed after a
+    # preemption, must start from an empty state
+    from spite_amd import Engine
+    define_parts()
+    t = tensors(5)
+    # every key stays visible here, so that requests grow until the pages run out
+    eng = Engine(spec=spec("full", 0), tensors=t, dtype="float32", page_size=4, num_pages=10, max_requests=3,
+                 max_batch_tokens=12)
+    prompts = [H.random_tokens(V, n, 30 + n) for n in (9, 14, 5, 11, 7, 3)]
+
+    def plain_generate(p, n):
+        toks = list(p)
+        for _ in range(n):
+            row = plain_toy(t, toks, "full", 0)[-1]
+            toks.append(int(row.argmax()))
+        return toks[len(p):]
+
+    stats = {}
+    got = eng.generate(prompts, max_tokens=7, temperature=0.0, eos_token_ids=[], stats=stats)
+    assert stats["preemptions"] > 0, "the pool was meant to be too small for three requests at once"
+    for p, g in zip(prompts, got):
+        assert g == plain_generate(p, 7)
+    eng.cache.check()

@@ -170,3 +170,52 @@ def test_mixed_checkpoint_keeps_32_bit_tensors(tmp_path):
     assert m.blocks[0].mixer.wo.dtype == torch.float32 and m.blocks[1].mixer.wo.dtype == torch.bfloat16
     assert m.blocks[0].norm1.weight.dtype == torch.float32 and m.blocks[0].ffn.w_router.dtype == torch.float32
     assert m.embed.dtype == torch.bfloat16
+
+
+def test_text_model_of_a_multimodal_folder(tmp_path):
+    # keys under text_config, tensors under language_model., other towers' tensors passed over;
+    # an unknown tensor under the text prefix is still an error, and so is a tower's tensor in a
+    # folder that says it is a text model
+    from spite_amd.weights.random_init import random_tensors
+    text = {k: v for k, v in TINY_A.items() if k != "architectures"}
+    cfg = {"architectures": ["Llama4ForConditionalGeneration"], "text_config": text}
+    d = str(tmp_path / "mm")
+    os.makedirs(d)
+    json.dump(cfg, open(os.path.join(d, "config.json"), "w"))
+    t = {"language_model." + k: v for k, v in random_tensors(TINY_A, 3).items()}
+    t["vision_model.patch_embedding.weight"] = torch.zeros(4, 4)
+    t["multi_modal_projector.linear_1.weight"] = torch.zeros(2, 2)
+    save_file(t, os.path.join(d, "model.safetensors"))
+    arch, c = read_config(d)
+    assert arch.name == "Llama4ForConditionalGeneration" and c.hidden_size == TINY_A["hidden_size"]
+    m = Model(arch.build_spec(c), Env(torch.float32, torch.device("cpu")))
+    load_weights(m, d, torch.float32)
+    assert m.embed.shape == (TINY_A["vocab_size"], TINY_A["hidden_size"])
+    t["language_model.model.layers.0.extra.weight"] = torch.zeros(1)
+    save_file(t, os.path.join(d, "model.safetensors"))
+    with pytest.raises(WeightsError, match="unexpected tensors: model.layers.0.extra.weight") as e:
+        load_weights(m, d, torch.float32)
+    assert "vision_model" not in str(e.value)
+    with pytest.raises(WeightsError, match="vision_model"):
+        load_weights(cpu_model(TINY_A), d, torch.float32)
+
+
+def test_one_binder_for_folders_tensors_in_memory_and_seeds():
+    from spite_amd.weights.loader import bind, DictSource, RandomSource
+    from spite_amd.weights.random_init import random_tensors, draw
+    m = cpu_model(TINY_B)
+    t = random_tensors(TINY_B, 9)
+    src = RandomSource(m.tensor_plan(), 9, 0.02, torch.float32)
+    assert sorted(src.names()) == sorted(t)
+    for n in t:
+        assert torch.equal(src.host(n), t[n])
+    bad = dict(t)
+    bad.pop("model.norm.weight")
+    bad["lm_head.weight"] = bad["lm_head.weight"][:-1]
+    bad["stray"] = torch.zeros(1)
+    with pytest.raises(WeightsError) as e:
+        bind(m, DictSource(bad), torch.float32)
+    msg = str(e.value)
+    assert "missing tensors: model.norm.weight" in msg and "unexpected tensors: stray" in msg and "lm_head.weight is" in msg
+    bind(m, DictSource(t), torch.float32)
+    assert torch.equal(m.final_norm.weight, t["model.norm.weight"])
