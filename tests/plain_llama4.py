@@ -101,8 +101,9 @@ def attn_temperature(positions: torch.Tensor, floor_scale: int, attn_scale: floa
 # --------------------------------------------------------------------------- attention
 
 
-def visible_mask(positions: torch.Tensor, kind: str, size: int = 0) -> torch.Tensor:
-    """``mask[p, j]`` true when the query at position p may read the key at position j.
+def visible_mask(positions: torch.Tensor, kind: str, size: int = 0, key_positions=None) -> torch.Tensor:
+    """``mask[p, j]`` true when the query at position p may read the key at position j
+    (``key_positions``: the keys' positions when they are not the queries' own).
 
     * ``full``: causal, j <= p (crates/spite-compute/src/flash_attn.rs:118-121).
     * ``window``: causal and among the last ``size`` rows, j > p - size
@@ -112,7 +113,7 @@ def visible_mask(positions: torch.Tensor, kind: str, size: int = 0) -> torch.Ten
       window "chunked", llama4.rs:6, but compute no chunks).
     """
     p = positions.to(torch.int64)[:, None]
-    j = positions.to(torch.int64)[None, :]
+    j = (positions if key_positions is None else key_positions).to(torch.int64)[None, :]
     m = j <= p
     if kind == "full":
         return m
@@ -141,6 +142,28 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: torch.Ten
         p = torch.exp(s - m)
         z = p.sum(-1, keepdim=True).clamp_min(1e-30)
         out[:, h, :] = (p / z) @ v[:, g, :]
+    return out
+
+
+def attention_rows(q, k, v, q_pos, kind: str, size: int = 0, key_start: int = 0, block: int = 1024) -> torch.Tensor:
+    """``attention`` for queries at positions ``q_pos`` (ascending) over keys at positions
+    ``key_start`` .. ``key_start + S - 1``, a block of queries at a time, so that a long
+    sequence never needs its whole score matrix at once.  A block only meets the keys from the
+    first one that its first query may read to its last query's own."""
+    out = torch.zeros_like(q)
+    S = k.shape[0]
+    key_pos = key_start + torch.arange(S)
+    for a in range(0, q.shape[0], block):
+        b = min(a + block, q.shape[0])
+        first, last = int(q_pos[a]), int(q_pos[b - 1])
+        lo = key_start
+        if kind == "chunk":
+            lo = max((first // size) * size, key_start)
+        elif kind == "window":
+            lo = max(first - size + 1, key_start)
+        lo, hi = lo - key_start, min(last + 1 - key_start, S)
+        mask = visible_mask(q_pos[a:b], kind, size, key_pos[lo:hi])
+        out[a:b] = attention(q[a:b], k[lo:hi], v[lo:hi], mask)
     return out
 
 
@@ -229,11 +252,16 @@ def layer_kinds(cfg: dict):
 
 
 def forward(cfg: dict, weights: dict, tokens, start_pos: int = 0, dtype=torch.float64,
-            visibility: str = "chunk", route_hints=None, hint_rel: float = 0.0, taken=None,
-            chosen=None) -> torch.Tensor:
+            visibility: str | None = None, route_hints=None, hint_rel: float = 0.0, taken=None,
+            chosen=None, rows=None) -> torch.Tensor:
     """Logits ``[T, V]`` of one whole sequence (crates/spite-models/src/llama/llama4.rs:74-283,
     layer-major instead of token-major; same arithmetic).  ``visibility`` of the rotating
-    layers: ``chunk`` (configuration) or ``window`` (what the reference computes)."""
+    layers: ``chunk`` (configuration) or ``window`` (what the reference computes); default: the
+    configuration's ``attention_local_kind``, else ``chunk``.  ``rows`` (ascending positions):
+    logits ``[len(rows), V]`` of these positions only; the last layer then computes nothing
+    else (every earlier layer feeds the keys of the next and stays whole)."""
+    if visibility is None:
+        visibility = cfg.get("attention_local_kind", "chunk")
     W = {k: v.to(dtype) for k, v in weights.items()}
     d = cfg["hidden_size"]
     H = cfg["num_attention_heads"]
@@ -249,40 +277,51 @@ def forward(cfg: dict, weights: dict, tokens, start_pos: int = 0, dtype=torch.fl
     pos = torch.arange(start_pos, start_pos + T)
 
     h = W["model.embed_tokens.weight"][tokens]                      # llama4.rs:118-119
-    for L in range(cfg["num_hidden_layers"]):
+    n_layers = cfg["num_hidden_layers"]
+    sel = None if rows is None else torch.as_tensor(list(rows), dtype=torch.int64) - start_pos
+    for L in range(n_layers):
         p = f"model.layers.{L}."
         n = rms_norm(h, W[p + "input_layernorm.weight"], eps)       # :126-127
-        q = (n @ W[p + "self_attn.q_proj.weight"].T).view(T, H, hd)  # :140-153
-        k = (n @ W[p + "self_attn.k_proj.weight"].T).view(T, G, hd)
+        k = (n @ W[p + "self_attn.k_proj.weight"].T).view(T, G, hd)  # :140-153
         v = (n @ W[p + "self_attn.v_proj.weight"].T).view(T, G, hd)
+        last = L == n_layers - 1 and sel is not None
+        if last:                                                    # only the wanted rows from here on
+            h, n, qpos = h[sel], n[sel], pos[sel]
+        else:
+            qpos = pos
+        q = (n @ W[p + "self_attn.q_proj.weight"].T).view(-1, H, hd)
         if uses_rope[L]:
-            q = apply_rope(q, pos, inv_freq, pairing)               # :157-160
+            q = apply_rope(q, qpos, inv_freq, pairing)              # :157-160
             k = apply_rope(k, pos, inv_freq, pairing)
             if cfg.get("use_qk_norm", True):
                 q = qk_l2_norm(q, eps)                              # :161-175
                 k = qk_l2_norm(k, eps)
-            mask = visible_mask(pos, visibility, C) if C else visible_mask(pos, "full")
+            kind, size = (visibility, C) if C else ("full", 0)
         else:
             if cfg.get("attn_temperature_tuning", True):
-                s = attn_temperature(pos, cfg.get("floor_scale", 8192), cfg.get("attn_scale", 0.1), dtype)
+                s = attn_temperature(qpos, cfg.get("floor_scale", 8192), cfg.get("attn_scale", 0.1), dtype)
                 q = q * s[:, None, None]                            # :178-183
-            mask = visible_mask(pos, "full")
-        o = attention(q, k, v, mask).reshape(T, H * hd)             # :198-201
+            kind, size = "full", 0
+        o = attention_rows(q, k, v, qpos, kind, size, start_pos).reshape(-1, H * hd)   # :198-201
         h = h + o @ W[p + "self_attn.o_proj.weight"].T              # :202-207
         n = rms_norm(h, W[p + "post_attention_layernorm.weight"], eps)  # :210-211
         f = p + "feed_forward."
         if is_moe[L]:
             took = []
+            hints = None if route_hints is None else route_hints.get(L)
+            if hints is not None and last:
+                hints = [hints[int(i)] for i in sel]
             y = moe_ffn(n, W[f + "router.weight"], W[f + "experts.gate_up_proj"], W[f + "experts.down_proj"],
                         W[f + "shared_expert.gate_proj.weight"], W[f + "shared_expert.up_proj.weight"],
                         W[f + "shared_expert.down_proj.weight"],    # :212-256
-                        None if route_hints is None else route_hints.get(L), hint_rel, took,
-                        None if chosen is None else chosen.setdefault(L, []))
+                        hints, hint_rel, took, None if chosen is None else chosen.setdefault(L, []))
             if taken is not None:
-                taken.extend((L, t) for t in took)
+                taken.extend((L, int(sel[t]) if last else t) for t in took)
         else:
             y = swiglu_mlp(n, W[f + "gate_proj.weight"], W[f + "up_proj.weight"], W[f + "down_proj.weight"])
         h = h + y                                                   # :272-274
+    if sel is not None and n_layers == 0:
+        h = h[sel]
     n = rms_norm(h, W["model.norm.weight"], eps)                    # :277-278
     head = W["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) else W["lm_head.weight"]
     return n @ head.T                                               # :279

@@ -79,6 +79,33 @@ def test_llama3_scaling():
         plain.rope_inv_freq(64, 10000.0, dict(sc, rope_type="yarn"))
 
 
+def test_llama3_scaling_is_continuous_and_monotonic_across_the_band():
+    # the reference has no frequency scaling, so nothing of its text or tests pins the blend
+    # between the two band edges (parity with the reference: unpinned).  What pins it here: the
+    # rescaled frequency must join the untouched short waves at one edge (s = 1) and the slowed
+    # long waves at the other (s = 0) without a jump, and the ratio to the plain frequency must
+    # fall steadily from 1 to 1/factor in between.  A blend with s and 1-s exchanged jumps at both
+    # edges and rises in between.  2,048 frequencies make the steps between neighbours small.
+    from spite_amd.parts.position import inv_frequencies
+    for factor, low, high, orig, theta in ((8.0, 1.0, 4.0, 64, 10000.0), (16.0, 1.0, 4.0, 8192, 500000.0)):
+        sc = dict(rope_type="llama3", factor=factor, low_freq_factor=low, high_freq_factor=high,
+                  original_max_position_embeddings=orig)
+        base = plain.rope_inv_freq(4096, theta, None)
+        ratio = plain.rope_inv_freq(4096, theta, sc) / base
+        wavelen = 2 * math.pi / base
+        band = (wavelen >= orig / high) & (wavelen <= orig / low)
+        assert 20 < int(band.sum()) < 2000
+        assert float(ratio.max()) == 1.0 and abs(float(ratio.min()) - 1.0 / factor) < 1e-12
+        steps = ratio[1:] - ratio[:-1]                       # frequencies fall with the index
+        assert (steps <= 1e-15).all(), "the ratio must never rise from short waves to long ones"
+        assert float(steps.abs().max()) < 3.0 * (1.0 - 1.0 / factor) / int(band.sum()), "a jump at a band edge"
+        # the engine's table is the same function
+        mine = torch.tensor(inv_frequencies(4096, theta, sc), dtype=torch.float64)
+        assert torch.allclose(mine, plain.rope_inv_freq(4096, theta, sc), rtol=1e-13, atol=0)
+        mine = torch.tensor(inv_frequencies(128, theta, sc), dtype=torch.float64)
+        assert torch.allclose(mine, plain.rope_inv_freq(128, theta, sc), rtol=1e-13, atol=0)
+
+
 def test_qk_norm_commutes_with_rotation():
     inv = plain.rope_inv_freq(8, 100.0, None)
     x = torch.randn(4, 3, 8, dtype=D)
@@ -282,6 +309,26 @@ def test_positions_shift_only_moves_chunks_and_temperature():
     # with chunks the shift moves the chunk borders and the logits change
     c = plain.forward(dict(cfg, attention_chunk_size=16), W, toks, start_pos=11)
     assert not torch.allclose(a, c, atol=1e-4)
+
+
+def test_wanted_rows_alone_and_blocks_of_queries_equal_the_whole():
+    from helpers import TINY_A, TINY_B, planted_tensors
+    for cfg, kind in ((TINY_A, None), (TINY_B, "window"), (dict(TINY_B, attention_local_kind="window"), None)):
+        W = {k: v.to(D) for k, v in planted_tensors(cfg, 3).items()}
+        toks = [(7 * i + 3) % cfg["vocab_size"] for i in range(75)]
+        whole = plain.forward(cfg, W, toks, start_pos=5, visibility=kind)
+        rows = [5, 6, 20, 36, 37, 52, 79]
+        some = plain.forward(cfg, W, toks, start_pos=5, visibility=kind, rows=rows)
+        assert torch.allclose(some, whole[[r - 5 for r in rows]], atol=1e-12)
+    g = torch.Generator().manual_seed(2)
+    q, k, v = (torch.randn(90, n, 8, generator=g, dtype=D) for n in (4, 2, 2))
+    pos = torch.arange(30, 120)
+    for kind, size in (("full", 0), ("chunk", 16), ("window", 11)):
+        whole = plain.attention(q, k, v, plain.visible_mask(pos, kind, size))
+        assert torch.allclose(plain.attention_rows(q, k, v, pos, kind, size, key_start=30, block=7), whole, atol=1e-12)
+        pick = torch.tensor([0, 3, 50, 89])
+        assert torch.allclose(plain.attention_rows(q[pick], k, v, pos[pick], kind, size, key_start=30, block=3),
+                              whole[pick], atol=1e-12)
 
 
 def test_layer_kinds():
