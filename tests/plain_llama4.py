@@ -65,14 +65,19 @@ def rope_inv_freq(head_dim: int, theta: float, scaling: dict | None) -> torch.Te
 
 
 def apply_rope(x: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor,
-               pairing: str = "half") -> torch.Tensor:
+               pairing: str = "half", angle_dtype=None) -> torch.Tensor:
     """crates/spite-rope/src/lib.rs:78-92 (rope_range): half-split pairs (i, i+hd/2):
     x_i' = x_i cos a - x_{i+half} sin a ; x_{i+half}' = x_i sin a + x_{i+half} cos a,
     a = pos * f_i; every head alike (lib.rs:69-71).  ``x`` is ``[T, heads, hd]``.
-    ``pairing="adjacent"`` pairs (2i, 2i+1) instead (not the reference's)."""
+    ``pairing="adjacent"`` pairs (2i, 2i+1) instead (not the reference's).
+    ``angle_dtype=torch.float32``: position, frequency and their product in 32-bit, as
+    lib.rs:82 forms them (``pos as f32 * freq``): at position p that angle is off by up to
+    p * 2^-24 rad, a thousandth at 17,000; sine and cosine of the rounded angle are then exact
+    here.  Default: everything in the dtype of ``x``."""
     hd = x.shape[-1]
     half = hd // 2
-    ang = positions.to(x.dtype)[:, None] * inv_freq.to(x.dtype)[None, :]  # [T, half]
+    adt = angle_dtype or x.dtype
+    ang = (positions.to(adt)[:, None] * inv_freq.to(adt)[None, :]).to(x.dtype)  # [T, half]
     cos = torch.cos(ang)[:, None, :]
     sin = torch.sin(ang)[:, None, :]
     out = torch.empty_like(x)
@@ -253,13 +258,14 @@ def layer_kinds(cfg: dict):
 
 def forward(cfg: dict, weights: dict, tokens, start_pos: int = 0, dtype=torch.float64,
             visibility: str | None = None, route_hints=None, hint_rel: float = 0.0, taken=None,
-            chosen=None, rows=None) -> torch.Tensor:
+            chosen=None, rows=None, rope_angle_dtype=None) -> torch.Tensor:
     """Logits ``[T, V]`` of one whole sequence (crates/spite-models/src/llama/llama4.rs:74-283,
     layer-major instead of token-major; same arithmetic).  ``visibility`` of the rotating
     layers: ``chunk`` (configuration) or ``window`` (what the reference computes); default: the
     configuration's ``attention_local_kind``, else ``chunk``.  ``rows`` (ascending positions):
     logits ``[len(rows), V]`` of these positions only; the last layer then computes nothing
-    else (every earlier layer feeds the keys of the next and stays whole)."""
+    else (every earlier layer feeds the keys of the next and stays whole).  ``rope_angle_dtype``:
+    see ``apply_rope``."""
     if visibility is None:
         visibility = cfg.get("attention_local_kind", "chunk")
     W = {k: v.to(dtype) for k, v in weights.items()}
@@ -291,8 +297,8 @@ def forward(cfg: dict, weights: dict, tokens, start_pos: int = 0, dtype=torch.fl
             qpos = pos
         q = (n @ W[p + "self_attn.q_proj.weight"].T).view(-1, H, hd)
         if uses_rope[L]:
-            q = apply_rope(q, qpos, inv_freq, pairing)              # :157-160
-            k = apply_rope(k, pos, inv_freq, pairing)
+            q = apply_rope(q, qpos, inv_freq, pairing, rope_angle_dtype)   # :157-160
+            k = apply_rope(k, pos, inv_freq, pairing, rope_angle_dtype)
             if cfg.get("use_qk_norm", True):
                 q = qk_l2_norm(q, eps)                              # :161-175
                 k = qk_l2_norm(k, eps)
