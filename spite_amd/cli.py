@@ -98,7 +98,10 @@ def cmd_random_model(args) -> int:
     from .weights.random_init import write_random_model
     with open(args.config, "r", encoding="utf-8") as fh:
         cfg = json.load(fh)
-    write_random_model(args.out, cfg, args.seed, args.std, args.dtype)
+    import torch
+    # the same numbers either way; a GPU draws them sooner
+    write_random_model(args.out, cfg, args.seed, args.std, args.dtype,
+                       device="cuda:0" if torch.cuda.is_available() else None)
     print(f"wrote {args.out}/config.json and model.safetensors (seed {args.seed}, std {args.std})")
     return 0
 

@@ -77,6 +77,17 @@ void attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_p
         bf16x8 vf[ND];
 #pragma unroll
         for (int d = 0; d < ND; ++d) vf[d] = __builtin_nontemporal_load((const bf16x8*)(vbase + d * 512));
+        if (key0 + 31 > p) {
+            // the block that holds the query's own key: the rows behind it still hold what the
+            // page's last owner left, and a probability of zero times a value that is not finite
+            // is not zero; those values are taken as zero (this lane's keys are key0 + qd*8 + e)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const bool dead = key0 + qd * 8 + e > p;
+#pragma unroll
+                for (int d = 0; d < ND; ++d) vf[d][e] = dead ? (bf16)0.f : vf[d][e];
+            }
+        }
 
         f32x4 s[2];
 #pragma unroll

@@ -211,6 +211,11 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
         // the running maxima move in the first blocks and seldom after: the output is rescaled
         // only when some column of the wave needs it (alpha is exactly 1 otherwise)
         const bool rescale = __any(alpha[0] != 1.0f || alpha[1] != 1.0f);
+        // keys behind the last query of the wave may lie behind the request's last position, where
+        // the page still holds what its last owner left; a probability of zero times a value that
+        // is not finite is not zero, so those values are taken as zero (the keys below a column's
+        // first visible one are the request's own, and finite)
+        const bool stale = key0 + PF_KEYS - 1 > pq_max;
 #pragma unroll
         for (int d = 0; d < ND; ++d) {
             if (rescale) {
@@ -219,7 +224,12 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
             }
 #pragma unroll
             for (int hh = 0; hh < 2; ++hh) {
-                const bf16x8 vf = *(const bf16x8*)(vb_ + (hh * ND + d) * 512);
+                bf16x8 vf = *(const bf16x8*)(vb_ + (hh * ND + d) * 512);
+                if (stale) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        vf[e] = key0 + hh * 32 + qd * 8 + e > pq_max ? (bf16)0.f : vf[e];
+                }
 #pragma unroll
                 for (int c = 0; c < 2; ++c)
                     o[c][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[c][hh], o[c][d], 0, 0, 0);

@@ -13,6 +13,7 @@ from __future__ import annotations
 import json
 import os
 import zlib
+from concurrent.futures import ThreadPoolExecutor
 from typing import Dict
 
 import numpy as np
@@ -84,21 +85,29 @@ def normal_numbers(n: int, seed: int, key: int, mean: float = 0.0, std: float = 
     base = (int(seed) * 0x9e3779b97f4a7c15 + int(key)) & _M64
     out = np.empty(n, dtype=np.float32)
     pairs = (n + 1) // 2
-    step = 1 << 20
+    step = 1 << 18
     with np.errstate(over="ignore"):
         base = _mix64(np.array([base], dtype=np.uint64))[0]
-        for j0 in range(0, pairs, step):
+
+    def block(j0):
+        with np.errstate(over="ignore"):
             j = np.arange(j0, min(j0 + step, pairs), dtype=np.uint64)
             h = _mix64(base + j * np.uint64(0xd1342543de82ef95))
-            u1 = ((h >> np.uint64(32)).astype(np.float64) + 1.0) * (1.0 / 4294967296.0)
-            r = np.sqrt(-2.0 * _exact_log(u1))
-            sn, cs = _exact_sincos_turns((h & np.uint64(0xffffffff)).astype(np.uint32))
-            z0 = (r * cs).astype(np.float32)
-            z1 = (r * sn).astype(np.float32)
-            both = np.empty(2 * len(j), dtype=np.float32)
-            both[0::2] = np.float32(std) * z0 + np.float32(mean)
-            both[1::2] = np.float32(std) * z1 + np.float32(mean)
-            out[2 * j0:2 * j0 + min(2 * len(j), n - 2 * j0)] = both[:n - 2 * j0]
+        u1 = ((h >> np.uint64(32)).astype(np.float64) + 1.0) * (1.0 / 4294967296.0)
+        r = np.sqrt(-2.0 * _exact_log(u1))
+        sn, cs = _exact_sincos_turns((h & np.uint64(0xffffffff)).astype(np.uint32))
+        both = np.empty(2 * len(j), dtype=np.float32)
+        both[0::2] = np.float32(std) * (r * cs).astype(np.float32) + np.float32(mean)
+        both[1::2] = np.float32(std) * (r * sn).astype(np.float32) + np.float32(mean)
+        out[2 * j0:2 * j0 + min(2 * len(j), n - 2 * j0)] = both[:n - 2 * j0]
+
+    starts = range(0, pairs, step)
+    if len(starts) > 1:          # numpy's loops release the interpreter's lock: blocks run side by side
+        with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:
+            list(pool.map(block, starts))
+    else:
+        for j0 in starts:
+            block(j0)
     return out
 
 
@@ -134,20 +143,22 @@ def draw_on_device(name: str, spec, seed: int, std: float, file_dtype: torch.dty
     return t if direct else t.to(file_dtype)
 
 
-def random_tensors(config: dict, seed: int, std: float = 0.02) -> Dict[str, torch.Tensor]:
-    """fp32 tensors by checkpoint name for ``config`` (a config.json dict)."""
+def random_tensors(config: dict, seed: int, std: float = 0.02, device=None) -> Dict[str, torch.Tensor]:
+    """fp32 tensors by checkpoint name for ``config`` (a config.json dict), on the host.  With a
+    GPU ``device`` they are drawn there and copied back: the same numbers, sooner."""
     from ..engine.model import Model
     arch, cfg = read_config(config)
     model = Model(arch.build_spec(cfg), Env(torch.float32, torch.device("cpu")))
     out = {}
     for fname, ps, _, _ in model.tensor_plan():
         if fname not in out:
-            out[fname] = draw(fname, ps, seed, std)
+            out[fname] = draw(fname, ps, seed, std) if device is None else \
+                draw_on_device(fname, ps, seed, std, torch.float32, device).cpu()
     return out
 
 
 def write_random_model(folder: str, config: dict, seed: int, std: float = 0.02, dtype: str | None = None,
-                       overrides: Dict[str, torch.Tensor] | None = None) -> str:
+                       overrides: Dict[str, torch.Tensor] | None = None, device=None) -> str:
     """Writes ``folder/config.json`` and ``folder/model.safetensors``; returns the folder.
 
     ``dtype`` of the stored matrices defaults to the config's ``torch_dtype``.  ``overrides``
@@ -157,7 +168,7 @@ def write_random_model(folder: str, config: dict, seed: int, std: float = 0.02, 
     if dtype not in _FILE_DTYPES:
         raise ValueError(f"dtype {dtype!r} (known: {sorted(_FILE_DTYPES)})")
     config["torch_dtype"] = dtype
-    tensors = random_tensors(config, seed, std)
+    tensors = random_tensors(config, seed, std, device)
     for name, t in (overrides or {}).items():
         if name not in tensors:
             raise KeyError(f"override for unknown tensor {name!r}")

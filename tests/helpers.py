@@ -49,7 +49,8 @@ def planted_tensors(cfg: dict, seed: int, std: float = 0.05, qk_gain: float = 2.
     that attention is far from uniform and the experts are told apart clearly: with plain
     N(0, std) weights a wrong mask or a wrong expert would change the logits very little."""
     from spite_amd.weights.random_init import random_tensors
-    t = random_tensors(cfg, seed, std)
+    # on a GPU box the kernel draws them (the same numbers as the host draws, sooner)
+    t = random_tensors(cfg, seed, std, device="cuda:0" if torch.cuda.is_available() else None)
     for name in list(t):
         if name.endswith("q_proj.weight") or name.endswith("k_proj.weight"):
             t[name] = t[name] * qk_gain

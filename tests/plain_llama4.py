@@ -192,11 +192,14 @@ def router_top1(x: torch.Tensor, w_router: torch.Tensor, hints=None, hint_rel: f
 
     ``hints[t]`` (optional) names the expert that another implementation chose for row t.
     Where it differs from the choice made here and the two logits lie within ``hint_rel``
-    times the largest |logit| of the row, the two experts are tied at that implementation's
+    times the size of the router's logits, the two experts are tied at that implementation's
     precision and the hint is followed (and counted in ``taken``); a hint further off is
-    ignored."""
+    ignored.  The size is the root mean square of all logits of the call: the error of a logit
+    that was computed from rounded inputs grows with the row's and the router's sizes, not with
+    the logit's own value, which cancellation can make as small as the gap itself."""
     logits = x @ w_router.T
     E = logits.shape[-1]
+    size = float(logits.pow(2).mean().sqrt())
     idx = torch.zeros(logits.shape[0], dtype=torch.int64)
     for t in range(logits.shape[0]):
         best = 0
@@ -205,7 +208,7 @@ def router_top1(x: torch.Tensor, w_router: torch.Tensor, hints=None, hint_rel: f
                 best = e
         if hints is not None and int(hints[t]) != best and 0 <= int(hints[t]) < E:
             gap = float(logits[t, best] - logits[t, int(hints[t])])
-            if gap <= hint_rel * float(logits[t].abs().max()):
+            if gap <= hint_rel * size:
                 best = int(hints[t])
                 if taken is not None:
                     taken.append(t)

@@ -57,3 +57,50 @@ def test_a_random_configuration_in_32_bit(seed, tmp_path):
         d, where = H.max_diff(rows, ref)
         assert d <= 3e-5 * scale, f"{label}: {d} at {where} (logits up to {scale}); {cfg}"
         del eng
+
+
+def random_config_bf16(seed: int):
+    """Sizes that the bfloat16 kernels of serving take: head sizes 64 and 128 with pages of 32 or
+    64 (MFMA attention; one seed in four draws another head size and runs the generic kernel),
+    widths that are multiples of 64 (weights in operand order), of 8 only (row-major MFMA
+    products) or of neither (the generic product)."""
+    r = np.random.RandomState(2000 + seed)
+    pick = lambda xs: r.choice(xs).item()
+    cfg, _ = random_config(seed)
+    G = pick([1, 2, 3])
+    cfg.update(hidden_size=pick([64, 128, 192, 256, 72, 136, 100]), num_key_value_heads=G,
+               num_attention_heads=G * pick([1, 2, 4, 5, 8]), head_dim=pick([64, 128, 64, 128, 64, 128, 32, 96]),
+               intermediate_size=pick([64, 128, 192, 72, 40]), intermediate_size_mlp=pick([64, 128, 80, 200]),
+               vocab_size=pick([128, 301, 1000, 2049]), attention_chunk_size=pick([32, 64, 96, 128, 100]),
+               tie_word_embeddings=bool(seed % 3 == 0), torch_dtype="bfloat16")
+    return cfg, pick([32, 64])
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_a_random_configuration_in_bfloat16(seed, tmp_path):
+    from spite_amd.engine.engine import Engine
+    cfg, page = random_config_bf16(seed)
+    weights = H.make_model(str(tmp_path), cfg, seed=seed, dtype="bfloat16")
+    lens = [int(n) for n in np.random.RandomState(seed).choice([1, 2, 17, 33, 70, 131, 200, 300], size=4)]
+    reqs = {f"r{i}": H.random_tokens(cfg["vocab_size"], n, seed * 10 + i) for i, n in enumerate(lens)}
+    up = lambda n: -(-n // page) * page
+    one, three = up(max(lens)), sum(sorted((up(n) for n in lens), reverse=True)[:3])
+    n_choices = sum(lens) * len(H.moe_layers(cfg))
+    for label, steps, pool in (("whole", H.schedule_whole(reqs), one), ("portions", H.schedule_portions(reqs), one),
+                               ("mixed", H.schedule_mixed(reqs, seed=seed, max_live=3), three)):
+        eng = Engine(str(tmp_path), dtype="bfloat16", page_size=page, cache_tokens=pool, max_requests=4)
+        routing = {}
+        rows = H.collect(steps, H.run_trace_inprocess(eng, steps, routing), cfg["vocab_size"])
+        assert all(eng.cache.free_pages(g) == eng.cache.total_pages(g) for g in range(eng.cache.n_groups()))
+        # the plain implementation follows the engine's expert where its own best two are tied at
+        # bfloat16's precision (see test_replay.py)
+        taken = []
+        ref = H.plain_logits(cfg, weights, reqs, H.routing_hints(cfg, steps, routing), 0.04, taken)
+        scale = max(float(np.abs(v).max()) for v in ref.values())
+        d, where = H.max_diff(rows, ref)
+        print(f"[bf16 config {seed}] {label}: {d / scale:.2%} of the scale at {where}; {len(taken)} of {n_choices} near ties; "
+              f"d={cfg['hidden_size']} hd={cfg['head_dim']} H={cfg['num_attention_heads']}/{cfg['num_key_value_heads']} "
+              f"F={cfg['intermediate_size']} V={cfg['vocab_size']} tied={cfg['tie_word_embeddings']} page={page}")
+        assert d <= 0.04 * scale, f"{label}: {d} at {where} (logits up to {scale}); {cfg}"
+        assert len(taken) <= max(3, 0.03 * n_choices)
+        del eng

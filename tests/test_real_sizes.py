@@ -4,9 +4,12 @@ tiny configurations of the other tests never reach the shapes that serving runs.
 (one with rotation and chunked attention, one without rotation over the whole context), four
 experts and a small vocabulary keep the model at 1.4 G parameters.  The bfloat16 engine is held
 against the 32-bit engine on the same stored weights, token by token, wherever both sent the
-token to the same experts (a near tie of two experts may fall differently in bfloat16)."""
+token to the same experts (a near tie of two experts may fall differently in bfloat16); the
+32-bit engine in turn is held against the plain implementation on the same folder, so the chain
+is plain <- 32-bit engine <- bfloat16 engine."""
 import numpy as np
 import pytest
+import torch
 
 import helpers as H
 
@@ -52,6 +55,17 @@ def test_bfloat16_against_32_bit_at_the_layer_sizes_of_scout(tmp_path):
     rows["float32"] = H.collect(steps, H.run_trace_inprocess(eng, steps, routing32), V)
     routes["float32"] = H.routing_hints(cfg, steps, routing32)
     del eng
+    # the plain implementation on the stored weights, in 32-bit (its products over widths of 5,120 to
+    # 16,384 then round as the engine's do, in another order: a relative 1e-5 of the logits' size)
+    weights = H.read_weights(folder)
+    reqs = {"a": a, "b": b[:70], "c": c}
+    ref = H.plain_logits(cfg, weights, reqs, dtype=torch.float32)
+    ref = {k: v for k, v in ref.items() if k in rows["float32"]}
+    scale = max(float(np.abs(v).max()) for v in ref.values())
+    d, where = H.max_diff(rows["float32"], ref)
+    print(f"[scout sizes] 32-bit engine against the plain implementation: max|diff| {d:.3e} at {where} (logits up to {scale:.2f})")
+    assert d <= 1e-4 * scale, (d, where)
+    del weights, ref
     eng = Engine(folder, dtype="bfloat16", page_size=64, cache_tokens=1024, max_requests=4, max_batch_tokens=512)
     own = {}
     H.run_trace_inprocess(eng, steps, own)

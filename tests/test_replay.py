@@ -21,10 +21,10 @@ TOL_F32_SCHEDULES = 2e-6
 TOL_BF16_REL = 0.04
 # bfloat16 only: the router's logits come from the same hidden states and carry the same
 # relative error as the output logits.  Where the plain implementation's best two router
-# logits of a token lie within that accepted error (this fraction of the token's largest
-# |logit|), the experts are tied at bfloat16's precision; the plain implementation then
-# follows the engine's choice, and the logits must agree within the tolerance under that
-# choice.  A choice further off is not followed and shows as a fault.
+# logits of a token lie within that accepted error (this fraction of the size of the layer's
+# router logits, their root mean square), the experts are tied at bfloat16's precision; the plain
+# implementation then follows the engine's choice, and the logits must agree within the
+# tolerance under that choice.  A choice further off is not followed and shows as a fault.
 HINT_REL = TOL_BF16_REL
 
 REQUESTS = {
