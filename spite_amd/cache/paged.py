@@ -40,9 +40,12 @@ class Group:
 
 class PagedCache:
     def __init__(self, needs: Sequence[CacheNeed], page_size: int, num_pages, max_requests: int,
-                 dtype: torch.dtype, device, allocate: bool = True):
+                 dtype: torch.dtype, device, allocate: bool = True, portion: Optional[int] = None):
         """``needs[i]``: what cache id i asks for.  ``num_pages``: pages of every group's pool
-        (an int), or one number per group in order of first use."""
+        (an int), or one number per group in order of first use.  With ``portion`` (the most
+        tokens of one request in a step) and one number for all, a group whose layers read a
+        chunk or a window only gets no more pages than ``max_requests`` requests can hold there
+        at a time, each a chunk or window and a portion (``peak_pages``), however long they are."""
         self.page_size, self.max_requests, self.dtype, self.device = int(page_size), int(max_requests), dtype, device
         self.groups: List[Group] = []
         self._group_of: Dict[int, int] = {}
@@ -67,13 +70,25 @@ class PagedCache:
         for g, n in zip(self.groups, pages):
             g.n_pages = n
         lib = hostlib.lib()
+        self._lib = lib
         kinds = hostlib.int_array(_KINDS[g.key[2]] for g in self.groups)
         spans = hostlib.int_array(g.key[3] for g in self.groups)
-        npg = hostlib.int_array(pages)
-        self._h = lib.spc_create(self.page_size, self.max_requests, n_groups, kinds, spans, npg)
-        if not self._h:
-            raise CacheError(hostlib.last_error())
-        self._lib = lib
+
+        def create():
+            h = lib.spc_create(self.page_size, self.max_requests, n_groups, kinds, spans, hostlib.int_array(pages))
+            if not h:
+                raise CacheError(hostlib.last_error())
+            return h
+        self._h = create()
+        if portion is not None and isinstance(num_pages, int):
+            cut = [min(n, self.max_requests * self.peak_pages(n * self.page_size, int(portion), g))
+                   for g, n in enumerate(pages)]
+            if cut != pages:
+                lib.spc_destroy(self._h)
+                pages = cut
+                for g, n in zip(self.groups, pages):
+                    g.n_pages = n
+                self._h = create()
         self._fresh_buf = (ctypes.c_int * (4 * self.max_requests + 4))()
         self.states: Dict[int, torch.Tensor] = {}
         if allocate:

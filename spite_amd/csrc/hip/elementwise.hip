@@ -759,3 +759,33 @@ extern "C" int spite_randn_fill(void* out, int dtype, size_t n, unsigned long lo
     SP_LAUNCH_CHECK("randn_fill");
     return 0;
 }
+
+// ------------------------------------------------------------------ what the memory gives
+// Reads `n16` 16-byte words once, with non-temporal loads, a contiguous piece per workgroup, and
+// leaves one float per wave, four per workgroup, in `out` (so that the loads cannot be dropped): the measure of
+// the read bandwidth that the weight-streaming kernels are held against.
+__global__ __launch_bounds__(256)
+void stream_read_kernel(const f32x4* __restrict__ p, size_t n16, size_t per_block, float* __restrict__ out) {
+    const size_t b0 = (size_t)blockIdx.x * per_block;
+    const size_t b1 = b0 + per_block < n16 ? b0 + per_block : n16;
+    f32x4 acc[4] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}};
+    size_t i = b0 + threadIdx.x;
+    for (; i + 768 < b1; i += 1024) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) acc[u] += __builtin_nontemporal_load(p + i + u * 256);
+    }
+    for (; i < b1; i += 256) acc[0] += __builtin_nontemporal_load(p + i);
+    const f32x4 a = acc[0] + acc[1] + acc[2] + acc[3];
+    const float v = wave_sum(a[0] + a[1] + a[2] + a[3]);
+    if ((threadIdx.x & 63) == 0) out[blockIdx.x * 4 + (threadIdx.x >> 6)] = v;
+}
+extern "C" int spite_stream_read(const void* p, size_t nbytes, float* out, int n_blocks, hipStream_t st) {
+    SP_REQUIRE(((uintptr_t)p & 15) == 0 && nbytes % 16 == 0, "stream_read: 16-byte words only");
+    SP_REQUIRE(n_blocks > 0, "stream_read: no workgroups");
+    const size_t n16 = nbytes / 16;
+    if (n16 == 0) return 0;
+    const size_t per = (n16 + n_blocks - 1) / n_blocks;
+    stream_read_kernel<<<n_blocks, 256, 0, st>>>((const f32x4*)p, n16, per, out);
+    SP_LAUNCH_CHECK("stream_read");
+    return 0;
+}

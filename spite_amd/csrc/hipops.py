@@ -51,6 +51,7 @@ def lib():
             "spite_gemm_tiled_split": [P, I, P, P, I, I, I, I, I, I, P, P],
             "spite_attn_prefill": [P, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, F, I, P],
             "spite_argmax_rows": [P, I, I, I, P, P, P, P],
+            "spite_stream_read": [P, c_size_t, P, I, P],
         }
         for name, args in sigs.items():
             fn = getattr(l, name)
@@ -420,20 +421,24 @@ def tiled_k_runs(M: int, N: int, K: int) -> int:
 
 
 def gemm_tiled(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None, glu=False,
-               shape=0):
+               shape=0, part=None):
     """Tiled bf16 MFMA product for many rows over weights in operand order (``operand_order``;
-    see gemm_tiled.hip); arguments as gemm_generic."""
+    see gemm_tiled.hip); arguments as gemm_generic.  ``part`` (fp32 ``[runs, M, N]``, plain
+    products only): the sum over k is cut into ``runs`` runs, each a workgroup of its own, whose
+    partial sums a second kernel adds: for few tiles (a short prompt against a narrow matrix),
+    see ``tiled_k_runs``."""
     rows_w = _gemm_checks(a, w, y, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, "gemm_tiled")
     if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise KernelError(f"gemm_tiled: bfloat16 operands only, got {a.dtype} and {w.dtype}")
-    runs = tiled_k_runs(M, N, K) if (offsets is None and a_rows is None and a_scale is None and y_rows is None
-                                     and not glu and shape == 0 and M > 0) else 1
-    if runs > 1:
-        # few tiles (a short prompt against a narrow matrix): the sum over k is cut into runs,
-        # each a workgroup of its own, and their partial sums are added by a second kernel
-        part = torch.empty((runs, M, N), dtype=torch.float32, device=a.device)
+    if part is not None:
+        if not (offsets is None and a_rows is None and a_scale is None and y_rows is None and not glu and shape == 0):
+            raise KernelError("gemm_tiled: partial sums are for plain products only")
+        if part.dim() != 3 or part.shape[1] != M or part.shape[2] != N or part.shape[0] < 2 or part.shape[0] > 8 \
+                or part.shape[0] * 4 > K // 64:
+            raise KernelError(f"gemm_tiled: partial sums {tuple(part.shape)} for M={M} N={N} K={K}")
         _check(lib().spite_gemm_tiled_split(_ptr(a, "a"), a.stride(0), _ptr(w, "w"), _ptr(y, "y"), dtype_code(y.dtype),
-                                            y.stride(0), M, N, K, runs, _ptr(part, "part"), _stream()), "gemm_tiled")
+                                            y.stride(0), M, N, K, part.shape[0], _ptr(part, "part", torch.float32),
+                                            _stream()), "gemm_tiled")
         return
     _check(lib().spite_gemm_tiled(
         _ptr(a, "a"), a.stride(0), _ptr(w, "w"), rows_w * K, _ptr(y, "y"), dtype_code(y.dtype), y.stride(0),
@@ -477,3 +482,14 @@ def argmax_rows(logits, out, scratch_v, scratch_i, n_rows=None):
     _check(lib().spite_argmax_rows(_ptr(logits, "logits", torch.float32), logits.stride(0), n, logits.shape[1],
                                    _ptr(scratch_v, "scratch_v", torch.float32), _ptr(scratch_i, "scratch_i", torch.int32),
                                    _ptr(out, "out", torch.int32), _stream()), "argmax")
+
+
+def stream_read(t, out):
+    """Reads the tensor ``t`` once with non-temporal loads, one contiguous piece per workgroup;
+    ``out`` (fp32, four elements per workgroup) receives sums that keep the loads alive.  For
+    measuring the memory's read bandwidth."""
+    nbytes = t.numel() * t.element_size()
+    if out.numel() < 4:
+        raise KernelError("stream_read: out holds four floats per workgroup")
+    _check(lib().spite_stream_read(_ptr(t, "t"), nbytes - nbytes % 16, _ptr(out, "out", torch.float32), out.numel() // 4,
+                                   _stream()), "stream_read")

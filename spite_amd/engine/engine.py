@@ -156,7 +156,8 @@ class Engine:
         if num_pages is None:
             tokens = cache_tokens if cache_tokens is not None else self.max_requests * 4096
             num_pages = max(1, -(-int(tokens) // self.page_size))
-        self.cache = PagedCache(needs, self.page_size, num_pages, self.max_requests, self.env.dtype, self.device)
+        self.cache = PagedCache(needs, self.page_size, num_pages, self.max_requests, self.env.dtype, self.device,
+                                portion=self.max_batch_tokens)
         if tensors is not None:
             self._source = DictSource(tensors)
         elif random_weights:

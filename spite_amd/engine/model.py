@@ -94,5 +94,5 @@ class Model:
         self.final_norm.forward(h, n, d1=pending[0] if len(pending) > 0 else None,
                                 d2=pending[1] if len(pending) > 1 else None, rows=ctx.logit_rows, write_h=False)
         logits = step_ws.take((ctx.n_out, self.spec.vocab_size), torch.float32)
-        linear(n, self.head, logits)
+        linear(n, self.head, logits, ws=ctx.ws)
         return logits

@@ -103,7 +103,7 @@ class Attention(Mixer):
         H, G, hd = self.H, self.G, self.hd
         ws = ctx.ws
         qkv = ws.take((T, (H + 2 * G) * hd), x.dtype)
-        linear(x, self.wqkv, qkv)
+        linear(x, self.wqkv, qkv, ws=ws)
         pe = self.position
         if not pe.fused:
             pe.transform(qkv, ctx.positions, H, G, hd)
@@ -136,5 +136,5 @@ class Attention(Mixer):
                                 cache.block_table, T, H, G, hd, cache.page_size, self.visibility, self.span,
                                 self.scale, kv_tiled=cache.tiled)
         out = ws.take((T, self.d), torch.float32)
-        linear(o, self.wo, out)
+        linear(o, self.wo, out, ws=ws)
         return out

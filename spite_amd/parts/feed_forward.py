@@ -43,9 +43,9 @@ class DenseGLU(FeedForward):
     def forward(self, x, x32, ctx, projected=None):
         T = x.shape[0]
         act = ctx.ws.take((T, self.F), x.dtype)
-        linear(x, self.w_gate_up, act, glu=True)
+        linear(x, self.w_gate_up, act, glu=True, ws=ctx.ws)
         y = ctx.ws.take((T, self.d), torch.float32)
-        linear(act, self.w_down, y)
+        linear(act, self.w_down, y, ws=ctx.ws)
         return (y,)
 
 
@@ -131,23 +131,23 @@ class MoeTop1Sigmoid(FeedForward):
             # read once per 16 of them there, so it runs as a plain product of its own (measured
             # at 64 tokens over 16 experts: 658 against 683 us for the two products of a layer)
             linear(x, self.w_gate_up, act, glu=True, offsets=offsets, n_groups=E, a_rows=src, a_scale=scale, rows=T,
-                   max_rows=16)
-            linear(x, self.w_gate_up.group(E), act[T:], glu=True, a_rows=src[T:], a_scale=scale[T:], rows=T)
-            linear(act, self.w_down, y, offsets=offsets, n_groups=E, y_rows=dst, rows=T, max_rows=16)
-            linear(act[T:], self.w_down.group(E), y, y_rows=dst[T:], rows=T)
+                   max_rows=16, ws=ws)
+            linear(x, self.w_gate_up.group(E), act[T:], glu=True, a_rows=src[T:], a_scale=scale[T:], rows=T, ws=ws)
+            linear(act, self.w_down, y, offsets=offsets, n_groups=E, y_rows=dst, rows=T, max_rows=16, ws=ws)
+            linear(act[T:], self.w_down.group(E), y, y_rows=dst[T:], rows=T, ws=ws)
             return (y[:T], y[T:])
         shape = grouped_tile_shape(T, E, groups - E) if T > SKINNY_MAX_ROWS else 0
         # every token goes to one expert: at most min(T, E) of their groups hold rows, and the shared one
         live = min(T, E) + (groups - E)
         linear(x, self.w_gate_up, act, glu=True, offsets=offsets, n_groups=groups, a_rows=src, a_scale=scale, rows=n,
-               max_rows=T, tile_shape=shape, live_groups=live)
+               max_rows=T, tile_shape=shape, live_groups=live, ws=ws)
         # slot s writes row dst[s]: rows [0,T) the routed result per token, rows [T,2T) the shared one
         # (the down product has too few column tiles for the larger row tile to pay)
         linear(act, self.w_down, y, offsets=offsets, n_groups=groups, y_rows=dst, rows=n, max_rows=T,
-               tile_shape=shape if shape == 4 else 0, live_groups=live)
+               tile_shape=shape if shape == 4 else 0, live_groups=live, ws=ws)
         if self.fused_shared:
             return (y[:T], y[T:])
         act_s = ws.take((T, self.Fs), x.dtype)
-        linear(x, self.ws_gate_up, act_s, glu=True)
-        linear(act_s, self.ws_down, y[T:])
+        linear(x, self.ws_gate_up, act_s, glu=True, ws=ws)
+        linear(act_s, self.ws_down, y[T:], ws=ws)
         return (y[:T], y[T:])

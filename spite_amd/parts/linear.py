@@ -13,8 +13,14 @@ import torch
 from ..csrc import hipops
 
 
-def _widen(x):
-    y = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+def _scratch(ws, shape, dtype, device):
+    """From the step's workspace when the caller has one (a warmed-up engine then allocates
+    nothing inside a step), else a fresh tensor."""
+    return ws.take(tuple(shape), dtype) if ws is not None else torch.empty(tuple(shape), dtype=dtype, device=device)
+
+
+def _widen(x, ws=None):
+    y = _scratch(ws, x.shape, torch.float32, x.device)
     hipops.convert(x, y)
     return y
 
@@ -76,13 +82,14 @@ def grouped_tile_shape(tokens: int, groups: int, whole_groups: int = 0) -> int:
 
 
 def linear(x, w, y, *, glu=False, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None, rows=None,
-           max_rows=None, tile_shape=0, live_groups=0):
+           max_rows=None, tile_shape=0, live_groups=0, ws=None):
     """y[r] = W . x[r] for ``rows`` rows (default: all of x; for a row list: its length).
 
     With ``glu`` the weight holds gate rows then up rows and y = silu(gate) * up.
     ``max_rows``: the most rows that one group can bring (default: ``rows``).
     ``tile_shape``: the prefill product's tile (``grouped_tile_shape``), 0 = the library's choice.
-    ``live_groups``: a promise that at most this many groups hold rows (0: none)."""
+    ``live_groups``: a promise that at most this many groups hold rows (0: none).
+    ``ws``: the workspace that temporaries (partial sums, widened rows) are taken from."""
     tiled = False
     if isinstance(w, Weight):
         w, tiled = w.data, w.tiled
@@ -98,8 +105,11 @@ def linear(x, w, y, *, glu=False, offsets=None, n_groups=1, a_rows=None, a_scale
                                a_scale=a_scale, y_rows=y_rows, glu=glu, max_rows=most, tiled=tiled,
                                live_groups=live_groups)
         elif tiled:
+            plain = offsets is None and a_rows is None and a_scale is None and y_rows is None and not glu and tile_shape == 0
+            runs = hipops.tiled_k_runs(M, N, K) if plain and M > 0 else 1
+            part = _scratch(ws, (runs, M, N), torch.float32, x.device) if runs > 1 else None
             hipops.gemm_tiled(x, w, y, M, N, K, offsets=offsets, n_groups=n_groups, a_rows=a_rows, a_scale=a_scale,
-                              y_rows=y_rows, glu=glu, shape=tile_shape)
+                              y_rows=y_rows, glu=glu, shape=tile_shape, part=part)
         else:
             hipops.gemm_mfma(x, w, y, M, N, K, offsets=offsets, n_groups=n_groups, a_rows=a_rows, a_scale=a_scale,
                              y_rows=y_rows, glu=glu)
@@ -107,12 +117,12 @@ def linear(x, w, y, *, glu=False, offsets=None, n_groups=1, a_rows=None, a_scale
     if tiled:
         raise hipops.KernelError("linear: a weight in operand order met an input that the MFMA products do not take")
     if w.dtype == torch.float32 and x.dtype != torch.float32:
-        x32 = _widen(x)
+        x32 = _widen(x, ws)
         if y.dtype == torch.float32:
             hipops.gemm_generic(x32, w, y, M, N, K, offsets=offsets, n_groups=n_groups, a_rows=a_rows,
                                 a_scale=a_scale, y_rows=y_rows, glu=glu)
         else:
-            y32 = torch.empty(y.shape, dtype=torch.float32, device=y.device)
+            y32 = _scratch(ws, y.shape, torch.float32, y.device)
             hipops.gemm_generic(x32, w, y32, M, N, K, offsets=offsets, n_groups=n_groups, a_rows=a_rows,
                                 a_scale=a_scale, y_rows=y_rows, glu=glu)
             hipops.convert(y32, y)

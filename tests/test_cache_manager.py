@@ -199,3 +199,24 @@ def test_slots_handed_out_are_reported_once_whoever_admitted_them():
     # released and admitted again between two steps: reported, once
     c.release(s)
     assert c.admit() == s and c.states[0][s].abs().sum() == 0
+
+
+def test_a_chunked_group_gets_no_more_pages_than_its_requests_can_hold():
+    needs = [CacheNeed(kv=KVNeed(8, 128, "chunk", 8192)), CacheNeed(kv=KVNeed(8, 128, "full")),
+             CacheNeed(kv=KVNeed(8, 128, "window", 100))]
+    c = PagedCache(needs, 64, 8 * 32768 // 64, 8, torch.bfloat16, torch.device("cpu"), allocate=False, portion=2048)
+    # a chunk of 8,192 and a portion of 2,048 are 160 pages of 64; the whole context stays with the full group
+    assert [c.total_pages(g) for g in range(3)] == [8 * 160, 8 * 512, 8 * c.peak_pages(32768, 2048, 2)]
+    assert c.peak_pages(32768, 2048, 2) == (100 + 2048 - 2) // 64 + 2
+    # eight requests of 30,000 tokens in portions of 2,048 never run out in the chunked group
+    slots = [c.admit() for _ in range(8)]
+    for at in range(0, 30000, 2048):
+        n = min(2048, 30000 - at)
+        for s in slots:
+            c.reserve(s, n)
+        for s in slots:
+            c.commit(s, n)
+    c.check()
+    # small pools are left as they are
+    small = PagedCache(needs[:2], 16, 8, 4, torch.float32, torch.device("cpu"), allocate=False, portion=2048)
+    assert [small.total_pages(g) for g in range(2)] == [8, 8]

@@ -259,8 +259,21 @@ def test_gemm_tiled_with_the_sum_over_k_cut_into_runs(M, N, K, out_dtype):
     assert tiled_k_runs(2048, 7168, 5120) == 1          # enough tiles: one run
 
     def fn(a, w, y, *args, **kw):
-        ops().gemm_tiled(a, ops().operand_order(w), y, *args, **kw)
+        part = torch.empty(runs, M, N, device=DEV) if runs > 1 else None
+        ops().gemm_tiled(a, ops().operand_order(w), y, *args, part=part, **kw)
     run_gemm(fn, torch.bfloat16, out_dtype, M, N, K)
+
+    # through the parts' entry, which takes the partial sums from the step's workspace
+    from spite_amd.parts.linear import linear, Weight
+    from spite_amd.engine.context import Workspace
+    a, w = rnd(M, K, dtype=torch.bfloat16, seed=1), rnd(N, K, dtype=torch.bfloat16, seed=2)
+    y, ws = torch.empty(M, N, dtype=out_dtype, device=DEV), Workspace(DEV, 1 << 24)
+    before = torch.cuda.memory_allocated()
+    linear(a, Weight(w), y, ws=ws) if M > 64 else None
+    want = a.float() @ w.float().T
+    if M > 64:
+        assert torch.cuda.memory_allocated() - before <= N * K * 2 + 512        # the weight's copy in operand order, no more
+        assert (y.float() - want).abs().max() <= 2e-2 * max(1.0, float(want.abs().max()))
 
 
 def test_gemm_tiled_refuses_what_it_cannot_do():
