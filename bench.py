@@ -112,14 +112,15 @@ def measured_peaks(dtype):
     from spite_amd.csrc import hipops
     dev = torch.device("cuda:0")
     buf = torch.empty(1 << 30, dtype=torch.float32, device=dev).normal_()
-    out = torch.zeros(4 * 2048, dtype=torch.float32, device=dev)
     best = 0.0
-    for _ in range(6):
-        torch.cuda.synchronize()
-        t = time.perf_counter()
-        hipops.stream_read(buf, out)
-        torch.cuda.synchronize()
-        best = max(best, buf.numel() * 4 / (time.perf_counter() - t))
+    for blocks in (512, 1024, 4096):
+        out = torch.zeros(8 * blocks, dtype=torch.float32, device=dev)
+        for _ in range(4):
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            hipops.stream_read(buf, out)
+            torch.cuda.synchronize()
+            best = max(best, buf.numel() * 4 / (time.perf_counter() - t))
     del buf
     res = {"hbm_read_GBps": round(best / 1e9, 1)}
     if dtype == "bf16":

@@ -110,8 +110,14 @@ void add_rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ d1,
                 if (out32) ((f32x4*)(out32 + (size_t)i * d))[c] = y;
                 if (proj) ((f32x4*)ys)[c] = y;
                 if (out) {
+                    if constexpr (sizeof(TO) == 2) {             // four bf16 in one 8-byte store (d % 4 == 0 here)
+                        bf16x4 o4;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) out[(size_t)i * d + 4 * c + e] = from_f32<TO>(y[e]);
+                        for (int e = 0; e < 4; ++e) o4[e] = (bf16)y[e];
+                        *(bf16x4*)((bf16*)out + (size_t)i * d + 4 * c) = o4;
+                    } else {
+                        ((f32x4*)((float*)out + (size_t)i * d))[c] = y;
+                    }
                 }
             }
         }
@@ -155,7 +161,7 @@ extern "C" int spite_add_rmsnorm(float* h, const float* d1, const float* d2, con
     SP_REQUIRE(sh <= 48 * 1024, "add_rmsnorm: rows of %d do not fit the projection's LDS", d);
     if (n_rows == 0) return 0;
     auto al = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
-    const bool vec = d % 4 == 0 && d <= 4 * NORM_NT * NORM_MAX_V && al(h) && al(d1) && al(d2) && al(w) && al(out32);
+    const bool vec = d % 4 == 0 && d <= 4 * NORM_NT * NORM_MAX_V && al(h) && al(d1) && al(d2) && al(w) && al(out32) && al(out);
 #define SP_NORM(TO) do { if (vec) add_rmsnorm_kernel<TO, true><<<n_rows, NORM_NT, sh, st>>>(h, d1, d2, w, (TO*)out, out32, rows, d, eps, write_h, proj, proj_out, P); \
         else add_rmsnorm_kernel<TO, false><<<n_rows, NORM_NT, sh, st>>>(h, d1, d2, w, (TO*)out, out32, rows, d, eps, write_h, proj, proj_out, P); } while (0)
     if (out_dtype == SP_F32) SP_NORM(float);
@@ -761,23 +767,24 @@ extern "C" int spite_randn_fill(void* out, int dtype, size_t n, unsigned long lo
 }
 
 // ------------------------------------------------------------------ what the memory gives
-// Reads `n16` 16-byte words once, with non-temporal loads, a contiguous piece per workgroup, and
-// leaves one float per wave, four per workgroup, in `out` (so that the loads cannot be dropped): the measure of
-// the read bandwidth that the weight-streaming kernels are held against.
-__global__ __launch_bounds__(256)
+// Reads `n16` 16-byte words once, with non-temporal loads, a contiguous piece per workgroup
+// (512 threads, four loads in flight each: the form that a sweep over threads, unrolling and
+// workgroups found fastest), and leaves one float per wave in `out` so that the loads cannot be
+// dropped: the measure of the read bandwidth that the weight-streaming kernels are held against.
+__global__ __launch_bounds__(512)
 void stream_read_kernel(const f32x4* __restrict__ p, size_t n16, size_t per_block, float* __restrict__ out) {
     const size_t b0 = (size_t)blockIdx.x * per_block;
     const size_t b1 = b0 + per_block < n16 ? b0 + per_block : n16;
     f32x4 acc[4] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}};
     size_t i = b0 + threadIdx.x;
-    for (; i + 768 < b1; i += 1024) {
+    for (; i + 3 * 512 < b1; i += 4 * 512) {
 #pragma unroll
-        for (int u = 0; u < 4; ++u) acc[u] += __builtin_nontemporal_load(p + i + u * 256);
+        for (int u = 0; u < 4; ++u) acc[u] += __builtin_nontemporal_load(p + i + u * 512);
     }
-    for (; i < b1; i += 256) acc[0] += __builtin_nontemporal_load(p + i);
+    for (; i < b1; i += 512) acc[0] += __builtin_nontemporal_load(p + i);
     const f32x4 a = acc[0] + acc[1] + acc[2] + acc[3];
     const float v = wave_sum(a[0] + a[1] + a[2] + a[3]);
-    if ((threadIdx.x & 63) == 0) out[blockIdx.x * 4 + (threadIdx.x >> 6)] = v;
+    if ((threadIdx.x & 63) == 0) out[blockIdx.x * 8 + (threadIdx.x >> 6)] = v;
 }
 extern "C" int spite_stream_read(const void* p, size_t nbytes, float* out, int n_blocks, hipStream_t st) {
     SP_REQUIRE(((uintptr_t)p & 15) == 0 && nbytes % 16 == 0, "stream_read: 16-byte words only");
@@ -785,7 +792,7 @@ extern "C" int spite_stream_read(const void* p, size_t nbytes, float* out, int n
     const size_t n16 = nbytes / 16;
     if (n16 == 0) return 0;
     const size_t per = (n16 + n_blocks - 1) / n_blocks;
-    stream_read_kernel<<<n_blocks, 256, 0, st>>>((const f32x4*)p, n16, per, out);
+    stream_read_kernel<<<n_blocks, 512, 0, st>>>((const f32x4*)p, n16, per, out);
     SP_LAUNCH_CHECK("stream_read");
     return 0;
 }

@@ -21,7 +21,10 @@
 //    one kilobyte in lane order).  A lane's loads are then the tile's 16 bytes at lane * 16,
 //    and k runs q*8 .. q*8+7 inside every 32: X is read to match.
 //
-// A row's sum runs over k in an order that does not depend on M or on the other rows.
+// Within one instantiation a row's sum runs over k in an order that does not depend on M or on
+// the other rows.  The caller picks the instantiation (S, and above 64 rows another kernel) from
+// the number of rows, so across step sizes a bfloat16 product agrees only to rounding; the
+// 32-bit path's products (gemm_generic.hip) give the same bits for every batch.
 #include "common.h"
 
 template <int R, int G, int S, int NW, bool GLU, bool TILED, typename TY>

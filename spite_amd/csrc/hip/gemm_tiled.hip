@@ -232,7 +232,25 @@ void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restri
         }
     }
 
-    // acc[a][b][i] of lane (r, q): column ncol[a] + q*4 + i, slot row0 + wm*WS + b*16 + r
+    // acc[a][b][i] of lane (r, q): column ncol[a] + q*4 + i, slot row0 + wm*WS + b*16 + r.  A lane's four
+    // columns go out in one store (8 bytes of bf16, 16 of fp32) where the row's address allows it.
+    const bool vec_ok = (ldy & 3) == 0 && (((uintptr_t)Y) & 15) == 0 && (N & 3) == 0;
+    auto put4 = [&](TY* dst, int n, const float (&v)[4]) {
+        if (vec_ok && n + 3 < N) {
+            if constexpr (sizeof(TY) == 2) {
+                bf16x4 o;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) o[i] = (bf16)v[i];
+                *(bf16x4*)(dst + n) = o;
+            } else {
+                *(f32x4*)(dst + n) = f32x4{v[0], v[1], v[2], v[3]};
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (n + i < N) dst[n + i] = from_f32<TY>(v[i]);
+        }
+    };
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
         const int s = row0 + wm * WS + b * 16 + r;
@@ -243,22 +261,21 @@ void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restri
         if (GLU) {
 #pragma unroll
             for (int a = 0; a < TG; ++a) {
-                const int n = ncol[a] + q * 4;
+                float v[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    if (n + i < N) {
-                        const float gv = acc[a][b][i] * sc, uv = acc[a + TG][b][i] * sc;
-                        yrow[n + i] = from_f32<TY>(gv / (1.0f + __expf(-gv)) * uv);
-                    }
+                    const float gv = acc[a][b][i] * sc, uv = acc[a + TG][b][i] * sc;
+                    v[i] = gv / (1.0f + __expf(-gv)) * uv;
                 }
+                put4(yrow, ncol[a] + q * 4, v);
             }
         } else {
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
-                const int n = ncol[a] + q * 4;
+                float v[4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (n + i < N) yrow[n + i] = from_f32<TY>(acc[a][b][i] * sc);
+                for (int i = 0; i < 4; ++i) v[i] = acc[a][b][i] * sc;
+                put4(yrow, ncol[a] + q * 4, v);
             }
         }
     }

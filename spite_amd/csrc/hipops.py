@@ -433,8 +433,8 @@ def gemm_tiled(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_sca
     if part is not None:
         if not (offsets is None and a_rows is None and a_scale is None and y_rows is None and not glu and shape == 0):
             raise KernelError("gemm_tiled: partial sums are for plain products only")
-        if part.dim() != 3 or part.shape[1] != M or part.shape[2] != N or part.shape[0] < 2 or part.shape[0] > 8 \
-                or part.shape[0] * 4 > K // 64:
+        if part.dim() != 3 or part.shape[1] != M or part.shape[2] != N or part.shape[0] < 2 or part.shape[0] > 32 \
+                or part.shape[0] * 2 > K // 64:
             raise KernelError(f"gemm_tiled: partial sums {tuple(part.shape)} for M={M} N={N} K={K}")
         _check(lib().spite_gemm_tiled_split(_ptr(a, "a"), a.stride(0), _ptr(w, "w"), _ptr(y, "y"), dtype_code(y.dtype),
                                             y.stride(0), M, N, K, part.shape[0], _ptr(part, "part", torch.float32),
@@ -486,10 +486,10 @@ def argmax_rows(logits, out, scratch_v, scratch_i, n_rows=None):
 
 def stream_read(t, out):
     """Reads the tensor ``t`` once with non-temporal loads, one contiguous piece per workgroup;
-    ``out`` (fp32, four elements per workgroup) receives sums that keep the loads alive.  For
+    ``out`` (fp32, eight elements per workgroup) receives sums that keep the loads alive.  For
     measuring the memory's read bandwidth."""
     nbytes = t.numel() * t.element_size()
-    if out.numel() < 4:
-        raise KernelError("stream_read: out holds four floats per workgroup")
-    _check(lib().spite_stream_read(_ptr(t, "t"), nbytes - nbytes % 16, _ptr(out, "out", torch.float32), out.numel() // 4,
+    if out.numel() < 8:
+        raise KernelError("stream_read: out holds eight floats per workgroup")
+    _check(lib().spite_stream_read(_ptr(t, "t"), nbytes - nbytes % 16, _ptr(out, "out", torch.float32), out.numel() // 8,
                                    _stream()), "stream_read")

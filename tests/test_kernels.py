@@ -268,11 +268,15 @@ def test_gemm_tiled_with_the_sum_over_k_cut_into_runs(M, N, K, out_dtype):
     from spite_amd.engine.context import Workspace
     a, w = rnd(M, K, dtype=torch.bfloat16, seed=1), rnd(N, K, dtype=torch.bfloat16, seed=2)
     y, ws = torch.empty(M, N, dtype=out_dtype, device=DEV), Workspace(DEV, 1 << 24)
-    before = torch.cuda.memory_allocated()
-    linear(a, Weight(w), y, ws=ws) if M > 64 else None
-    want = a.float() @ w.float().T
     if M > 64:
-        assert torch.cuda.memory_allocated() - before <= N * K * 2 + 512        # the weight's copy in operand order, no more
+        weight = Weight(w)
+        linear(a, weight, y, ws=ws)
+        assert ws._off >= (runs * M * N * 4 if runs > 1 else 0)    # the partial sums came from the workspace
+        ws.reset()
+        before = torch.cuda.memory_allocated()
+        linear(a, weight, y, ws=ws)
+        assert torch.cuda.memory_allocated() == before          # and a warmed-up call allocates nothing
+        want = a.float() @ w.float().T
         assert (y.float() - want).abs().max() <= 2e-2 * max(1.0, float(want.abs().max()))
 
 
