@@ -31,7 +31,9 @@
 
 #define TLD 72             // padded row of the X tile in LDS, in elements (64 k + 8)
 
-template <int WN, int WM, int NB, bool GLU, typename TY, bool NTW>
+// GROUPED: the grouped form (row lists per group); apart from what it leaves out of the plain
+// product's code, it gives the two forms names of their own in a trace.
+template <int WN, int WM, int NB, bool GLU, typename TY, bool NTW, bool GROUPED>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restrict__ W, long w_group_stride,
                        TY* __restrict__ Y, int ldy, int M, int N, int K,
@@ -55,7 +57,7 @@ void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restri
     const int ks = unit_id % k_splits, tile_id = unit_id / k_splits;
     const int tile_m = tile_id % m_tiles, tile_n = tile_id / m_tiles;
     int g = 0, row0, row_end = M;
-    if (offsets) {
+    if (GROUPED) {
         if (!sp_find_tile(offsets, n_groups, BM, tile_m, g, row0, row_end)) return;
     } else {
         row0 = tile_m * BM;
@@ -294,14 +296,23 @@ static int launch_tiled_kernel(const void* X, int ldx, const void* W, long w_gro
     const size_t sh = (size_t)2 * BM * TLD * sizeof(bf16);
     static bool allowed = false;        // one flag per instantiation; more LDS than the default limit for WM = 2
     if (!allowed) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<WN, WM, NB, GLU, TY, NTW>,
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<WN, WM, NB, GLU, TY, NTW, true>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)sh);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<WN, WM, NB, GLU, TY, NTW, false>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)sh);
         SP_REQUIRE(e == hipSuccess, "gemm_tiled: %zu bytes of LDS refused: %s", sh, hipGetErrorString(e));
         allowed = true;
     }
-    gemm_tiled_kernel<WN, WM, NB, GLU, TY, NTW><<<dim3((m_tiles * n_tiles * k_splits + 7) / 8 * 8), 512, sh, st>>>(
-        (const bf16*)X, ldx, (const bf16*)W, w_group_stride, (TY*)Y, ldy, M, N, K, offsets, n_groups, a_rows, a_scale,
-        y_rows, m_tiles, n_tiles, k_splits, split_stride);
+    const dim3 grid((m_tiles * n_tiles * k_splits + 7) / 8 * 8);
+    if (offsets)
+        gemm_tiled_kernel<WN, WM, NB, GLU, TY, NTW, true><<<grid, 512, sh, st>>>(
+            (const bf16*)X, ldx, (const bf16*)W, w_group_stride, (TY*)Y, ldy, M, N, K, offsets, n_groups, a_rows, a_scale,
+            y_rows, m_tiles, n_tiles, k_splits, split_stride);
+    else
+        gemm_tiled_kernel<WN, WM, NB, GLU, TY, NTW, false><<<grid, 512, sh, st>>>(
+            (const bf16*)X, ldx, (const bf16*)W, w_group_stride, (TY*)Y, ldy, M, N, K, offsets, n_groups, a_rows, a_scale,
+            y_rows, m_tiles, n_tiles, k_splits, split_stride);
     SP_LAUNCH_CHECK("gemm_tiled");
     return 0;
 }
