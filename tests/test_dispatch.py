@@ -34,18 +34,25 @@ def test_runs_of_a_split_product_are_never_empty():
 def test_the_benchmark_counts_what_a_query_can_see():
     import importlib.util
     import os
+    from spite_amd.config import read_config
     spec = importlib.util.spec_from_file_location("bench", os.path.join(os.path.dirname(os.path.dirname(__file__)), "bench.py"))
     bench = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(bench)
-    for T, past, span in ((5, 0, None), (7, 9, None), (6, 0, 4), (10, 13, 8), (3, 7, 8), (20, 30, 16)):
-        brute = sum(1 for p in range(past, past + T) for j in range(p + 1) if span is None or j >= (p // span) * span)
-        assert bench.visible_pairs(T, past, span) == brute
-    cfg = dict(bench.SCOUT)
+    # pairs of (query, key) of a portion, against a count by hand: layers that rotate read their chunk or window
+    for kind in ("chunk", "window"):
+        for T, past, span in ((5, 0, 64), (7, 9, 64), (6, 0, 4), (10, 13, 8), (3, 7, 8), (20, 30, 16)):
+            cfg = dict(bench.TINY, num_hidden_layers=4, no_rope_layers=[1, 1, 0, 1], attention_chunk_size=span,
+                       attention_local_kind=kind)
+            sizes = bench.Sizes(read_config(cfg)[1], 2)
+            first = (lambda p: (p // span) * span) if kind == "chunk" else (lambda p: max(p - span + 1, 0))
+            local = sum(1 for p in range(past, past + T) for j in range(p + 1) if j >= first(p))
+            full = sum(p + 1 for p in range(past, past + T))
+            assert sizes.pairs(T, past) == 3 * local + full, (kind, T, past, span)
+    sizes = bench.Sizes(read_config(dict(bench.SCOUT, no_rope_layers=None))[1], 2)
     # more context costs more bytes on every layer below a chunk, only on every fourth above it
-    a = bench.decode_bytes(cfg, 48, 8, 4096, 6.4)
-    b = bench.decode_bytes(cfg, 48, 8, 4097, 6.4)
-    c = bench.decode_bytes(cfg, 48, 8, 32768, 6.4)
-    d = bench.decode_bytes(cfg, 48, 8, 32769, 6.4)
+    a, b = sizes.decode_bytes(8, 4096, 6.4), sizes.decode_bytes(8, 4097, 6.4)
+    c, d = sizes.decode_bytes(8, 32768, 6.4), sizes.decode_bytes(8, 32769, 6.4)
     kv_token = 2 * 8 * 128 * 2
     assert b - a == 8 * 48 * kv_token and d - c == 8 * 48 * kv_token
-    assert bench.decode_bytes(cfg, 48, 8, 8192, 6.4) < bench.decode_bytes(cfg, 48, 8, 8191, 6.4)   # a new chunk begins
+    assert sizes.decode_bytes(8, 8192, 6.4) < sizes.decode_bytes(8, 8191, 6.4)   # a new chunk begins
+    assert len(sizes.full_layers) == 12 and sizes.n_moe == 48
