@@ -259,10 +259,33 @@ def test_a_toy_architecture_is_registered_by_name_and_served_from_a_folder(tmp_p
     assert json.load(open(os.path.join(folder, "config.json")))["architectures"] == ["ToyWindowLM"]
     eng = Engine(folder, dtype="float32", page_size=4, cache_tokens=128, max_requests=3)
     assert eng.spec.architecture == "ToyWindowLM" and len(eng.spec.order) == 3
-    # the head is tied to the embedding; whole, token by token and mixed agree (no plain
-    # implementation of this model exists: the engine is held against itself)
+    # the head is tied to the embedding; the folder's tensors through a plain float64 reading of
+    # the same list of parts, then whole, token by token and mixed against each other
+    import plain_llama4 as plain
+    W = H.read_weights(folder)
+
+    def plain_toy_window(tokens):
+        T, d, heads, hd = len(tokens), raw["width"], raw["heads"], raw["width"] // raw["heads"]
+        pos = torch.arange(T)
+        h = W["toy.words"][torch.tensor(tokens)]
+        mask = plain.visible_mask(pos, "window", raw["window"])
+        for L in (0, 1, 1):                                           # the order list: block 1 twice
+            p = f"toy.{L}."
+            ln = lambda x, n: F.layer_norm(x, (d,), W[p + n + ".w"], W[p + n + ".b"], raw["ln_eps"])
+            n = ln(h, "ln1")
+            s = (1 + 0.5 * torch.cos(pos.double()[:, None] * W[p + "freq"][None, :]))[:, None, :]
+            q = (n @ W[p + "q_proj"].T).view(T, heads, hd) * s
+            k = (n @ W[p + "k_proj"].T).view(T, 1, hd) * s
+            v = (n @ W[p + "v_proj"].T).view(T, 1, hd)
+            h = h + plain.attention(q, k, v, mask).reshape(T, d) @ W[p + "o_proj"].T
+            h = h + plain.swiglu_mlp(ln(h, "ln2"), W[p + "gate_proj"], W[p + "up_proj"], W[p + "down_proj"])
+        return (plain.rms_norm(h, W["toy.out_norm"], 1e-5) @ W["toy.words"].T).float().numpy()
+
     reqs = {"x": H.random_tokens(77, 21, 1), "y": H.random_tokens(77, 10, 2)}
     whole = H.collect(H.schedule_whole(reqs), H.run_trace_inprocess(eng, H.schedule_whole(reqs)), 77)
+    ref = {(rid, i): row for rid, toks in reqs.items() for i, row in enumerate(plain_toy_window(toks))}
+    d, where = H.max_diff(whole, ref)
+    assert d < 2e-4 * max(1.0, max(abs(v).max() for v in ref.values())), (d, where)
     for steps in (H.schedule_tail_one_by_one(reqs, tail=6), H.schedule_mixed(reqs, seed=2, max_live=2)):
         d, where = H.max_diff(H.collect(steps, H.run_trace_inprocess(eng, steps), 77), whole)
         assert d < 1e-4, (d, where)
@@ -277,4 +300,7 @@ def test_a_toy_architecture_is_registered_by_name_and_served_from_a_folder(tmp_p
     assert abs(rows["long"][("long", 39)] - rows["other"][("other", 39)]).max() < 1e-5
     assert abs(rows["long"][("long", 24)] - rows["other"][("other", 24)]).max() > 1e-3
     out = eng.generate([long[:7]], max_tokens=5)
-    assert len(out[0]) == 5 and all(0 <= t < 77 for t in out[0])
+    toks = list(long[:7])
+    for _ in range(5):
+        toks.append(int(plain_toy_window(toks)[-1].argmax()))
+    assert out[0] == toks[7:]
