@@ -9,7 +9,6 @@ import torch
 from ..csrc import hipops
 from ..parts import base as P
 from ..parts.base import ParamSpec, PartSpec, CacheNeed
-from ..parts.linear import linear, Weight
 from .context import Env, Workspace, StepContext
 
 
@@ -18,8 +17,15 @@ class Model:
         self.spec, self.env = spec, env
         self.blocks = [P.build("block", PartSpec(bs.kind, {"spec": bs}), env) for bs in spec.blocks]
         self.final_norm = P.build("norm", spec.final_norm, env)
-        self.embed: Optional[torch.Tensor] = None
-        self.head: Optional[torch.Tensor] = None
+        V, d = spec.vocab_size, spec.hidden_size
+        self.embedding_spec = spec.embedding or PartSpec("token_table", {"vocab_size": V, "width": d},
+                                                         {"weight": spec.embed_name})
+        self.head_spec = spec.head or PartSpec("linear_head", {"vocab_size": V, "width": d, "tied": spec.head_name is None},
+                                               {} if spec.head_name is None else {"weight": spec.head_name})
+        if spec.embedding is None and spec.embed_name is None:
+            raise ValueError("the model spec names neither an embedding part nor the embedding table's tensor")
+        self.embedding = P.build("embedding", self.embedding_spec, env)
+        self.head = P.build("head", self.head_spec, env)
         for i, call in enumerate(spec.order):
             if not 0 <= call.block < len(self.blocks):
                 raise ValueError(f"layer call {i} names block {call.block} of {len(self.blocks)}")
@@ -33,17 +39,21 @@ class Model:
             if not call.write and (call.cache not in writers or writers[call.cache] > i):
                 raise ValueError(f"layer call {i} reads cache {call.cache} before any call has written it")
         self._writers = writers
-        self.graph_safe = all(b.graph_safe for b in self.blocks) and self.final_norm.graph_safe
+        self.graph_safe = all(b.graph_safe for b in self.blocks) and self.final_norm.graph_safe \
+            and self.embedding.graph_safe and self.head.graph_safe
         self.step_arrays = tuple(sorted({a for b in self.blocks for a in b.step_arrays}))
 
     # ------------------------------------------------------------------ tensors
     def tensor_plan(self) -> List[Tuple[str, ParamSpec, object, str]]:
         """(checkpoint name, spec, owning part, local name) of every tensor of the model."""
         plan = []
-        V, d = self.spec.vocab_size, self.spec.hidden_size
-        plan.append((self.spec.embed_name, ParamSpec((V, d)), self, "embed"))
-        if self.spec.head_name is not None:
-            plan.append((self.spec.head_name, ParamSpec((V, d)), self, "head"))
+        ends = [("embedding", self.embedding, self.embedding_spec), ("head", self.head, self.head_spec)]
+        for what, part, pspec in ends:
+            for local, ps in part.params().items():
+                if local not in pspec.names or pspec.names[local] is None:
+                    raise KeyError(f"the {what} {pspec.kind!r} declares tensor {local!r} but its spec names no "
+                                   f"checkpoint tensor for it")
+                plan.append((pspec.names[local], ps, part, local))
         for local, ps in self.final_norm.params().items():
             plan.append((self.spec.final_norm.names[local], ps, self.final_norm, local))
         for block in self.blocks:
@@ -55,17 +65,8 @@ class Model:
                     plan.append((pspec.names[local], ps, part, local))
         return plan
 
-    def load(self, tensors: Dict[str, torch.Tensor]):   # the model's own two tensors
-        if "embed" in tensors:
-            self.embed = tensors["embed"].contiguous()
-        if "head" in tensors:
-            self.head = Weight(tensors["head"])
-
     def finish_loading(self):
-        if self.embed is None:
-            raise RuntimeError("model has no embedding table")
-        if self.spec.head_name is None:       # tied: the table stays row-major, the embedding reads its rows
-            self.head = self.embed
+        self.head.tie(self.embedding)
 
     def cache_needs(self) -> List[Optional[CacheNeed]]:
         n = max((c.cache for c in self.spec.order), default=-1) + 1
@@ -80,7 +81,8 @@ class Model:
         ``[n_out, V]`` at ``ctx.logit_rows``."""
         T, d = ctx.T, self.spec.hidden_size
         h = step_ws.take((T, d), torch.float32)
-        hipops.embed(ctx.token_ids, self.embed, h)
+        ctx.ws = arenas[0]
+        self.embedding.forward(ctx.token_ids, h, ctx)
         pending = ()
         for i, call in enumerate(self.spec.order):
             ctx.ws = arenas[i % 2]
@@ -94,5 +96,5 @@ class Model:
         self.final_norm.forward(h, n, d1=pending[0] if len(pending) > 0 else None,
                                 d2=pending[1] if len(pending) > 1 else None, rows=ctx.logit_rows, write_h=False)
         logits = step_ws.take((ctx.n_out, self.spec.vocab_size), torch.float32)
-        linear(n, self.head, logits, ws=ctx.ws)
+        self.head.forward(n, logits, ctx)
         return logits

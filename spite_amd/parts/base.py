@@ -78,12 +78,14 @@ class ModelSpec:
     blocks: List[BlockSpec]
     order: List[LayerCall]
     final_norm: PartSpec
-    embed_name: str
-    head_name: Optional[str]     # None: the embedding table is the output matrix
+    embed_name: Optional[str] = None     # shorthand for embedding = token_table under this tensor name
+    head_name: Optional[str] = None      # shorthand for head = linear_head; None: tied to the embedding's table
     eos_token_ids: Tuple[int, ...] = ()
     max_position: int = 1 << 20  # the default context limit of generation (the step function itself has none)
     strip_prefixes: Tuple[str, ...] = ("language_model.",)   # taken off the checkpoint's tensor names
     ignore_prefixes: Tuple[str, ...] = ()   # tensors of the checkpoint that belong to no part of this model
+    embedding: Optional[PartSpec] = None    # other kinds of the two ends than the shorthands above name
+    head: Optional[PartSpec] = None
 
 
 class Part:
@@ -156,6 +158,24 @@ class FeedForward(Part):
         raise NotImplementedError
 
 
+class Embedding(Part):
+    #: the table [V, d] after loading, for a head that is tied to it (None if there is none)
+    table = None
+
+    def forward(self, token_ids, h, ctx) -> None:
+        """h (fp32 [T,d]) = the residual stream's first value for the step's token ids (int32 [T])."""
+        raise NotImplementedError
+
+
+class Head(Part):
+    def tie(self, embedding: Embedding) -> None:
+        """Called once after loading, with the model's embedding (a tied head takes its table)."""
+
+    def forward(self, x, logits, ctx) -> None:
+        """logits (fp32 [n,V]) from the final norm's rows x ([n,d] in the run's dtype)."""
+        raise NotImplementedError
+
+
 class Block(Part):
     def forward(self, h, pending, ctx, cache):
         """Runs the layer on the residual stream h (fp32 [T,d]); ``pending`` are up to two
@@ -185,7 +205,7 @@ def step_array_builder(name: str) -> Callable:
 
 # ----------------------------------------------------------------------------- registries
 _REGISTRIES: Dict[str, Dict[str, Callable]] = {
-    "norm": {}, "position": {}, "mixer": {}, "ffn": {}, "block": {},
+    "norm": {}, "position": {}, "mixer": {}, "ffn": {}, "block": {}, "embedding": {}, "head": {},
 }
 
 

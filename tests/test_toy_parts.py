@@ -304,3 +304,71 @@ def test_a_toy_architecture_is_registered_by_name_and_served_from_a_folder(tmp_p
     for _ in range(5):
         toks.append(int(plain_toy_window(toks)[-1].argmax()))
     assert out[0] == toks[7:]
+
+
+def test_other_ends_of_a_model_an_embedding_with_a_scale_and_a_head_with_a_cap_and_a_bias():
+    """The two ends are parts too: an embedding that scales its rows by sqrt(width) and a head that
+    adds a bias and caps the logits with a tanh, defined here, beside the built-in layers."""
+    import math
+    from spite_amd import Engine
+    from spite_amd.parts import Embedding, Head, ParamSpec, PartSpec, BlockSpec, LayerCall, ModelSpec, register
+
+    @register("embedding", "toy_scaled_table")
+    class ScaledTable(Embedding):
+        def __init__(self, env, vocab_size, width):
+            self.V, self.d = vocab_size, width
+
+        def params(self):
+            return {"weight": ParamSpec((self.V, self.d))}
+
+        def load(self, t):
+            self.table = t["weight"]
+
+        def forward(self, token_ids, h, ctx):
+            h.copy_(self.table[token_ids.long()].float() * math.sqrt(self.d))
+
+    @register("head", "toy_capped_head")
+    class CappedHead(Head):
+        def __init__(self, env, vocab_size, width, cap):
+            self.V, self.d, self.cap = vocab_size, width, cap
+
+        def params(self):
+            return {"weight": ParamSpec((self.V, self.d)), "bias": ParamSpec((self.V,), kind="vector", init="zeros")}
+
+        def load(self, t):
+            self.w, self.b = t["weight"], t["bias"]
+
+        def forward(self, x, logits, ctx):
+            logits.copy_(self.cap * torch.tanh((x.float() @ self.w.float().T + self.b) / self.cap))
+
+    rms = lambda name: PartSpec("rms", {"width": D, "eps": 1e-5}, {"weight": name})
+    attn = PartSpec("attention", dict(hidden_size=D, n_heads=HEADS, n_kv_heads=KV, head_dim=HD,
+                                      position=PartSpec("rotary", {"head_dim": HD, "theta": 100.0})),
+                    {k: f"b1.attn.{k}" for k in ("q_proj", "k_proj", "v_proj", "o_proj")})
+    dense = PartSpec("dense_glu", {"hidden_size": D, "intermediate_size": 40},
+                     {k: f"b1.ffn.{k}" for k in ("gate_proj", "up_proj", "down_proj")})
+    sp = ModelSpec("ToyEnds", V, D, [BlockSpec("prenorm", rms("b1.n1"), attn, rms("b1.n2"), dense)], [LayerCall(0, 0)], rms("final"),
+                   embedding=PartSpec("toy_scaled_table", {"vocab_size": V, "width": D}, {"weight": "embed"}),
+                   head=PartSpec("toy_capped_head", {"vocab_size": V, "width": D, "cap": 2.0}, {"weight": "head", "bias": "head_bias"}))
+    t = {k: v for k, v in tensors(3).items() if k in ("embed", "head", "final") or k.startswith("b1.")}
+    t["head_bias"] = torch.linspace(-1, 1, V)
+    eng = Engine(spec=sp, tensors=t, dtype="float32", page_size=4, cache_tokens=64, max_requests=2)
+    import plain_llama4 as plain
+    W = {k: v.double() for k, v in t.items()}
+    toks = H.random_tokens(V, 19, 6)
+    T, pos = len(toks), torch.arange(len(toks))
+    h = W["embed"][torch.tensor(toks)] * math.sqrt(D)
+    n = plain.rms_norm(h, W["b1.n1"], 1e-5)
+    inv = plain.rope_inv_freq(HD, 100.0, None)
+    q = plain.apply_rope((n @ W["b1.attn.q_proj"].T).view(T, HEADS, HD), pos, inv)
+    k = plain.apply_rope((n @ W["b1.attn.k_proj"].T).view(T, KV, HD), pos, inv)
+    v = (n @ W["b1.attn.v_proj"].T).view(T, KV, HD)
+    h = h + plain.attention(q, k, v, plain.visible_mask(pos, "full", 0)).reshape(T, HEADS * HD) @ W["b1.attn.o_proj"].T
+    h = h + plain.swiglu_mlp(plain.rms_norm(h, W["b1.n2"], 1e-5), W["b1.ffn.gate_proj"], W["b1.ffn.up_proj"], W["b1.ffn.down_proj"])
+    ref = (2.0 * torch.tanh((plain.rms_norm(h, W["final"], 1e-5) @ W["head"].T + W["head_bias"]) / 2.0)).float().numpy()
+    reqs = {"x": toks}
+    for steps in (H.schedule_whole(reqs), H.schedule_portions(reqs, sizes=(3, 2, 7, 2))):
+        got = H.collect(steps, H.run_trace_inprocess(eng, steps), V)
+        err = max(abs(got[("x", i)] - ref[i]).max() for i in range(T))
+        assert err < 1e-4, err
+    assert abs(ref).max() > 1.5            # the cap is felt

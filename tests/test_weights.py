@@ -81,7 +81,7 @@ def test_loading_binds_every_tensor(tmp_path):
     m = cpu_model(TINY_A)
     load_weights(m, d, torch.float32)
     w = load_file(os.path.join(d, "model.safetensors"))
-    assert torch.equal(m.embed, w["model.embed_tokens.weight"]) and torch.equal(m.head.data, w["lm_head.weight"])
+    assert torch.equal(m.embedding.table, w["model.embed_tokens.weight"]) and torch.equal(m.head.weight.data, w["lm_head.weight"])
     att = m.blocks[2].mixer
     assert not att.wqkv.tiled                     # operand order is for bfloat16 matrices on the GPU
     assert torch.equal(att.wqkv.data[:64], w["model.layers.2.self_attn.q_proj.weight"])
@@ -146,7 +146,7 @@ def test_tied_embeddings_need_no_head(tmp_path):
     assert "lm_head.weight" not in load_file(os.path.join(d, "model.safetensors"))
     m = cpu_model(cfg)
     load_weights(m, d, torch.float32)
-    assert m.head is m.embed
+    assert m.head.weight is m.embedding.table
 
 
 def test_resident_dtypes():
@@ -169,7 +169,7 @@ def test_mixed_checkpoint_keeps_32_bit_tensors(tmp_path):
     load_weights(m, d, torch.bfloat16)
     assert m.blocks[0].mixer.wo.dtype == torch.float32 and m.blocks[1].mixer.wo.dtype == torch.bfloat16
     assert m.blocks[0].norm1.weight.dtype == torch.float32 and m.blocks[0].ffn.w_router.dtype == torch.float32
-    assert m.embed.dtype == torch.bfloat16
+    assert m.embedding.table.dtype == torch.bfloat16
 
 
 def test_text_model_of_a_multimodal_folder(tmp_path):
@@ -190,7 +190,7 @@ def test_text_model_of_a_multimodal_folder(tmp_path):
     assert arch.name == "Llama4ForConditionalGeneration" and c.hidden_size == TINY_A["hidden_size"]
     m = Model(arch.build_spec(c), Env(torch.float32, torch.device("cpu")))
     load_weights(m, d, torch.float32)
-    assert m.embed.shape == (TINY_A["vocab_size"], TINY_A["hidden_size"])
+    assert m.embedding.table.shape == (TINY_A["vocab_size"], TINY_A["hidden_size"])
     t["language_model.model.layers.0.extra.weight"] = torch.zeros(1)
     save_file(t, os.path.join(d, "model.safetensors"))
     with pytest.raises(WeightsError, match="unexpected tensors: model.layers.0.extra.weight") as e:
