@@ -175,12 +175,15 @@ extern "C" int spite_add_rmsnorm(float* h, const float* d1, const float* d2, con
 // ------------------------------------------------------------------ rotation, qk-norm, temperature, cache write
 // One wave per (token, head).  Heads [0,H) are queries, [H,H+G) keys, [H+G,H+2G) values of
 // the fused projection row.  Queries and keys: rotate by pos*inv_freq (if use_rope), then
-// the weightless RMS norm over the head (if use_norm); queries alone are then multiplied by
-// ln(floor((pos+1)/floor_scale)+1)*attn_scale+1 (if use_temp).  Keys and values go to the
-// request's page: cache row = slot_map[t] = page*page_size + offset.  Key pages are laid out
-// [page][kv head][offset][hd]; value pages transposed, [page][kv head][hd][offset], so that
-// the attention kernels read eight consecutive keys of one value column in one load (the
+// the RMS norm over the head (if use_norm; weightless, or times w_q / w_k if given); queries alone
+// are then multiplied by ln(floor((pos+1)/floor_scale)+1)*attn_scale+1 (if use_temp).  Keys and
+// values go to the request's page: cache row = slot_map[t] = page*page_size + offset.  Key pages
+// are laid out [page][kv head][offset][hd]; value pages transposed, [page][kv head][hd][offset],
+// so that the attention kernels read eight consecutive keys of one value column in one load (the
 // layout of an MFMA operand whose sum runs over keys).
+// Options that other architectures' attention needs: `rot` < hd rotates the first `rot`
+// elements of a head only (pairs (i, i + rot/2), or adjacent ones) and passes the rest through;
+// `norm_first` norms (and weights) before the rotation instead of after it.
 #define SP_MAX_PAIRS 4   // head sizes up to 512
 // Four waves a workgroup; a wave takes `hpw` heads of one token in turn and computes the
 // token's sines and cosines once for all of them.
@@ -191,20 +194,23 @@ void rope_kvwrite_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
                          const int* __restrict__ positions, const int* __restrict__ slot_map,
                          const float* __restrict__ inv_freq, int H, int G, int hd, int ps,
                          int use_rope, int adjacent, int use_norm, float norm_eps,
-                         int use_temp, int floor_scale, float attn_scale, int n_heads, int hpw, int kv_tiled) {
+                         int use_temp, int floor_scale, float attn_scale, int n_heads, int hpw, int kv_tiled,
+                         int rot, const float* __restrict__ w_q, const float* __restrict__ w_k, int norm_first) {
     const int t = blockIdx.x;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int half = hd >> 1;
+    const int half = hd >> 1, rhalf = rot >> 1;
     const int row_w = (H + 2 * G) * hd;
     const int pos = positions[t];
     const int slot = slot_map ? slot_map[t] : -1;
+    // pair i of a head: the rotating pairs first (i < rot/2), then the elements behind `rot` two by two
+    auto first_of = [&](int i) { return adjacent ? 2 * i : (i < rhalf ? i : rot + (i - rhalf)); };
+    auto second_of = [&](int i) { return adjacent ? 2 * i + 1 : (i < rhalf ? i + rhalf : rot + (i - rhalf) + (half - rhalf)); };
     float sn[SP_MAX_PAIRS], cs[SP_MAX_PAIRS];
-    if (use_rope) {
 #pragma unroll
-        for (int u = 0; u < SP_MAX_PAIRS; ++u) {
-            const int i = lane + u * 64;
-            if (i < half) sincosf((float)pos * inv_freq[i], &sn[u], &cs[u]);
-        }
+    for (int u = 0; u < SP_MAX_PAIRS; ++u) {
+        const int i = lane + u * 64;
+        sn[u] = 0.f; cs[u] = 1.f;                    // pairs that do not rotate
+        if (use_rope && i < rhalf) sincosf((float)pos * inv_freq[i], &sn[u], &cs[u]);
     }
     float temp = 1.f;
     if (use_temp) temp = logf((float)((pos + 1) / floor_scale) + 1.0f) * attn_scale + 1.0f;
@@ -233,16 +239,15 @@ void rope_kvwrite_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
             dst = k_pages + (page * G + g) * (size_t)ps * hd;
             if (!kv_tiled) dst += (size_t)off * hd;
         }
+        const float* wn = is_q ? w_q : w_k;
         float x0[SP_MAX_PAIRS], x1[SP_MAX_PAIRS];
         float ss = 0.f;
 #pragma unroll
         for (int u = 0; u < SP_MAX_PAIRS; ++u) {
             const int i = lane + u * 64;
             if (i < half) {
-                const int i0 = adjacent ? 2 * i : i;
-                const int i1 = adjacent ? 2 * i + 1 : i + half;
-                float a = to_f32<T>(src[i0]), b = to_f32<T>(src[i1]);
-                if (use_rope) {
+                float a = to_f32<T>(src[first_of(i)]), b = to_f32<T>(src[second_of(i)]);
+                if (use_rope && !norm_first) {
                     const float ra = a * cs[u] - b * sn[u];
                     const float rb = a * sn[u] + b * cs[u];
                     a = ra; b = rb;
@@ -256,15 +261,23 @@ void rope_kvwrite_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
             ss = wave_sum(ss);
             scale = 1.0f / sqrtf(ss / (float)hd + norm_eps);
         }
-        if (is_q) scale *= temp;
+        const float last = is_q ? temp : 1.f;
 #pragma unroll
         for (int u = 0; u < SP_MAX_PAIRS; ++u) {
             const int i = lane + u * 64;
             if (i < half) {
-                const int i0 = adjacent ? 2 * i : i;
-                const int i1 = adjacent ? 2 * i + 1 : i + half;
-                dst[tiled_k ? sp_k_index(off, i0, hd, true) : (size_t)i0] = from_f32<T>(x0[u] * scale);
-                dst[tiled_k ? sp_k_index(off, i1, hd, true) : (size_t)i1] = from_f32<T>(x1[u] * scale);
+                const int i0 = first_of(i), i1 = second_of(i);
+                float a = x0[u] * scale, b = x1[u] * scale;
+                if (use_norm && wn) { a *= wn[i0]; b *= wn[i1]; }
+                if (use_rope && norm_first) {
+                    const float ra = a * cs[u] - b * sn[u];
+                    const float rb = a * sn[u] + b * cs[u];
+                    a = ra; b = rb;
+                }
+                if (!use_norm || wn || norm_first) { a *= last; b *= last; }
+                else { a = x0[u] * (scale * last); b = x1[u] * (scale * last); }   // the plain case's one product
+                dst[tiled_k ? sp_k_index(off, i0, hd, true) : (size_t)i0] = from_f32<T>(a);
+                dst[tiled_k ? sp_k_index(off, i1, hd, true) : (size_t)i1] = from_f32<T>(b);
             }
         }
     }
@@ -374,11 +387,14 @@ void rope_kvwrite_vec_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ q_
     }
 }
 
+// `rotary_dim`: how many leading elements of a head rotate (0 or hd: all); `w_q`, `w_k`: weights of the
+// qk-norm ([hd] fp32) or null for the weightless norm; `norm_first`: norm before the rotation.
 extern "C" int spite_rope_kvwrite(const void* qkv, void* q_out, void* k_pages, void* v_pages, int dtype,
                                   const int* positions, const int* slot_map, const float* inv_freq,
                                   int T, int H, int G, int hd, int page_size, int use_rope, int adjacent,
                                   int use_norm, float norm_eps, int use_temp, int floor_scale,
-                                  float attn_scale, int write_kv, int kv_tiled, hipStream_t st) {
+                                  float attn_scale, int write_kv, int kv_tiled, int rotary_dim, const float* w_q,
+                                  const float* w_k, int norm_first, hipStream_t st) {
     SP_REQUIRE(T >= 0 && H > 0 && G > 0 && hd > 0 && page_size > 0, "rope_kvwrite: bad sizes");
     SP_REQUIRE(hd % 2 == 0 && hd <= 128 * SP_MAX_PAIRS, "rope_kvwrite: head size %d must be even and <= %d",
                hd, 128 * SP_MAX_PAIRS);
@@ -388,12 +404,16 @@ extern "C" int spite_rope_kvwrite(const void* qkv, void* q_out, void* k_pages, v
     SP_REQUIRE(!write_kv || slot_map, "rope_kvwrite: writing the cache needs the rows' slots");
     SP_REQUIRE(!kv_tiled || (dtype == SP_BF16 && hd % 32 == 0 && page_size % 32 == 0),
                "rope_kvwrite: pages in operand order are bfloat16 with head size %d and page size %d multiples of 32", hd, page_size);
+    const int rot = rotary_dim > 0 ? rotary_dim : hd;
+    SP_REQUIRE(rot % 2 == 0 && rot <= hd, "rope_kvwrite: %d rotating elements of a head of %d", rot, hd);
+    SP_REQUIRE((!w_q && !w_k) || use_norm, "rope_kvwrite: norm weights without a norm");
     if (T == 0) return 0;
     const int n_heads = write_kv ? H + 2 * G : H;
     const int hpw = T >= 256 ? 4 : 1;            // many tokens: fewer, longer workgroups
     const int lph = hd / 8;                      // lanes a head in the 8-byte kernel
     auto al8 = [](const void* p) { return ((uintptr_t)p & 7) == 0; };
-    if (dtype == SP_BF16 && hd % 8 == 0 && lph >= 1 && lph <= 64 && (lph & (lph - 1)) == 0 && al8(qkv) && al8(q_out)
+    const bool plain = rot == hd && !w_q && !w_k && !norm_first;     // what the 8-byte kernel knows
+    if (plain && dtype == SP_BF16 && hd % 8 == 0 && lph >= 1 && lph <= 64 && (lph & (lph - 1)) == 0 && al8(qkv) && al8(q_out)
         && al8(k_pages) && (page_size % 4 == 0 || !write_kv)) {
         const int hpi = 64 / lph;
         dim3 grid(T, (n_heads + 4 * hpw * hpi - 1) / (4 * hpw * hpi));
@@ -407,11 +427,11 @@ extern "C" int spite_rope_kvwrite(const void* qkv, void* q_out, void* k_pages, v
     if (dtype == SP_F32)
         rope_kvwrite_kernel<float><<<grid, 256, 0, st>>>((const float*)qkv, (float*)q_out, (float*)k_pages,
             (float*)v_pages, positions, slot_map, inv_freq, H, G, hd, page_size, use_rope, adjacent, use_norm,
-            norm_eps, use_temp, floor_scale, attn_scale, n_heads, hpw, kv_tiled);
+            norm_eps, use_temp, floor_scale, attn_scale, n_heads, hpw, kv_tiled, rot, w_q, w_k, norm_first);
     else if (dtype == SP_BF16)
         rope_kvwrite_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)qkv, (bf16*)q_out, (bf16*)k_pages,
             (bf16*)v_pages, positions, slot_map, inv_freq, H, G, hd, page_size, use_rope, adjacent, use_norm,
-            norm_eps, use_temp, floor_scale, attn_scale, n_heads, hpw, kv_tiled);
+            norm_eps, use_temp, floor_scale, attn_scale, n_heads, hpw, kv_tiled, rot, w_q, w_k, norm_first);
     else return sp_fail("rope_kvwrite: unknown dtype %d", dtype);
     SP_LAUNCH_CHECK("rope_kvwrite");
     return 0;

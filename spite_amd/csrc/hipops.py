@@ -35,7 +35,7 @@ def lib():
         sigs = {
             "spite_embed": [P, P, I, P, I, I, I, P],
             "spite_add_rmsnorm": [P, P, P, P, P, I, P, P, I, I, F, I, P, P, I, P],
-            "spite_rope_kvwrite": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, I, I, F, I, I, P],
+            "spite_rope_kvwrite": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, I, I, F, I, I, I, P, P, I, P],
             "spite_router_top1": [P, P, P, P, P, I, I, I, P],
             "spite_moe_plan": [P, P, P, P, P, P, P, I, I, I, P],
             "spite_convert": [P, I, P, I, c_size_t, P],
@@ -150,10 +150,12 @@ def add_rmsnorm(h, w, eps, out=None, out32=None, d1=None, d2=None, rows=None, n_
 
 def rope_kvwrite(qkv, q_out, k_pages, v_pages, positions, slot_map, inv_freq, H, G, hd, page_size, *,
                  use_rope, adjacent, use_norm, norm_eps, use_temp, floor_scale, attn_scale, write_kv=True,
-                 kv_tiled=False):
-    """Rotation, weightless qk-norm and temperature of the fused projection's rows; keys and
-    values go to their cache rows.  qkv [T,(H+2G)*hd]; q_out [T,H*hd]; key pages
-    [n_pages, G, page_size, hd], value pages [n_pages, G, hd, page_size]."""
+                 kv_tiled=False, rotary_dim=None, norm_weight_q=None, norm_weight_k=None, norm_first=False):
+    """Rotation, qk-norm and temperature of the fused projection's rows; keys and values go to
+    their cache rows.  qkv [T,(H+2G)*hd]; q_out [T,H*hd]; key pages [n_pages, G, page_size, hd],
+    value pages [n_pages, G, hd, page_size].  ``rotary_dim``: only the first so many elements of a
+    head rotate (default: all); ``norm_weight_q`` / ``norm_weight_k`` (fp32 [hd]): the norm's
+    weights (default: weightless); ``norm_first``: the norm comes before the rotation."""
     T = qkv.shape[0]
     if qkv.shape[1] != (H + 2 * G) * hd:
         raise KernelError(f"rope_kvwrite: qkv {tuple(qkv.shape)} for H={H} G={G} hd={hd}")
@@ -163,15 +165,25 @@ def rope_kvwrite(qkv, q_out, k_pages, v_pages, positions, slot_map, inv_freq, H,
         if slot_map.numel() < T:
             raise KernelError("rope_kvwrite: slot map too small")
         _check_pages(k_pages, v_pages, G, page_size, hd, "rope_kvwrite")
-    if use_rope and inv_freq.numel() != hd // 2:
-        raise KernelError("rope_kvwrite: frequency table does not match the head size")
+    rot = hd if rotary_dim is None else int(rotary_dim)
+    if hd % 2:
+        raise KernelError(f"rope_kvwrite: head size {hd} must be even")
+    if rot % 2 or not 0 < rot <= hd:
+        raise KernelError(f"rope_kvwrite: {rot} rotating elements of a head of {hd}")
+    if use_rope and inv_freq.numel() != rot // 2:
+        raise KernelError("rope_kvwrite: frequency table does not match the rotating part of the head")
+    for name, w in (("norm_weight_q", norm_weight_q), ("norm_weight_k", norm_weight_k)):
+        if w is not None and (w.numel() != hd or not use_norm):
+            raise KernelError(f"rope_kvwrite: {name} of {w.numel()} for heads of {hd} (norm {'on' if use_norm else 'off'})")
     dt = qkv.dtype
     _check(lib().spite_rope_kvwrite(
         _ptr(qkv, "qkv"), _ptr(q_out, "q_out", dt), _ptr(k_pages, "k_pages", dt, not write_kv),
         _ptr(v_pages, "v_pages", dt, not write_kv), dtype_code(dt), _ptr(positions, "positions", torch.int32),
         _ptr(slot_map, "slot_map", torch.int32, not write_kv), _ptr(inv_freq, "inv_freq", torch.float32, not use_rope),
         T, H, G, hd, page_size, int(use_rope), int(adjacent), int(use_norm), float(norm_eps), int(use_temp),
-        int(floor_scale), float(attn_scale), int(write_kv), int(bool(kv_tiled)), _stream()), "rope_kvwrite")
+        int(floor_scale), float(attn_scale), int(write_kv), int(bool(kv_tiled)), rot,
+        _ptr(norm_weight_q, "norm_weight_q", torch.float32, True), _ptr(norm_weight_k, "norm_weight_k", torch.float32, True),
+        int(bool(norm_first)), _stream()), "rope_kvwrite")
 
 
 def router_top1(x32, w_router, expert, weight, logits_out=None):

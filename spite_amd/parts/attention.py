@@ -45,7 +45,8 @@ class Attention(Mixer):
     step_arrays = (TAIL,)
 
     def __init__(self, env, hidden_size, n_heads, n_kv_heads, head_dim, position, visibility="full", span=0,
-                 qk_norm=False, qk_norm_eps=1e-5, temperature=None, softmax_scale=None):
+                 qk_norm=False, qk_norm_eps=1e-5, temperature=None, softmax_scale=None, qk_norm_weighted=False,
+                 qk_norm_first=False):
         if n_heads % n_kv_heads:
             raise ValueError(f"attention: {n_heads} heads over {n_kv_heads} kv heads")
         if visibility not in ("full", "chunk", "window"):
@@ -56,6 +57,10 @@ class Attention(Mixer):
         self.d, self.H, self.G, self.hd = int(hidden_size), int(n_heads), int(n_kv_heads), int(head_dim)
         self.visibility, self.span = visibility, int(span or 0)
         self.qk_norm, self.qk_norm_eps = bool(qk_norm), float(qk_norm_eps)
+        # the head norm's weights ([hd] each for queries and keys) and its place: after the rotation
+        # (Llama 4, weightless) or before it
+        self.qk_norm_weighted, self.qk_norm_first = bool(qk_norm_weighted) and self.qk_norm, bool(qk_norm_first)
+        self.w_qnorm = self.w_knorm = None
         self.temperature = temperature            # None or (floor_scale, attn_scale)
         self.scale = float(softmax_scale) if softmax_scale is not None else 1.0 / math.sqrt(self.hd)
         self.position = build_part("position", position, env)
@@ -66,6 +71,9 @@ class Attention(Mixer):
         d, H, G, hd = self.d, self.H, self.G, self.hd
         p = {"q_proj": ParamSpec((H * hd, d)), "k_proj": ParamSpec((G * hd, d)),
              "v_proj": ParamSpec((G * hd, d)), "o_proj": ParamSpec((d, H * hd))}
+        if self.qk_norm_weighted:
+            p["q_norm"] = ParamSpec((hd,), kind="vector", init="ones")
+            p["k_norm"] = ParamSpec((hd,), kind="vector", init="ones")
         p.update({f"position.{k}": v for k, v in self.position.params().items()})
         return p
 
@@ -76,6 +84,8 @@ class Attention(Mixer):
         dt = torch.float32 if len(dts) > 1 else dts.pop()
         self.wqkv = Weight(torch.cat([t["q_proj"].to(dt), t["k_proj"].to(dt), t["v_proj"].to(dt)], dim=0))
         self.wo = Weight(t["o_proj"])
+        if self.qk_norm_weighted:
+            self.w_qnorm, self.w_knorm = t["q_norm"].contiguous(), t["k_norm"].contiguous()
         self.position.load({k[len("position."):]: v for k, v in t.items() if k.startswith("position.")})
 
     def cache_need(self):
@@ -114,7 +124,8 @@ class Attention(Mixer):
                             H, G, hd, cache.page_size, use_rope=ka["use_rope"], adjacent=ka["adjacent"],
                             use_norm=self.qk_norm, norm_eps=self.qk_norm_eps, use_temp=temp is not None,
                             floor_scale=temp[0] if temp else 1, attn_scale=temp[1] if temp else 0.0,
-                            write_kv=cache.write, kv_tiled=cache.tiled)
+                            write_kv=cache.write, kv_tiled=cache.tiled, rotary_dim=ka.get("rotary_dim"),
+                            norm_weight_q=self.w_qnorm, norm_weight_k=self.w_knorm, norm_first=self.qk_norm_first)
         o = ws.take((T, H * hd), x.dtype)
         # the MFMA kernels read pages in operand order (bfloat16, sizes in multiples of 32)
         mfma = cache.tiled and hd in (64, 128)

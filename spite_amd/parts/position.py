@@ -43,19 +43,23 @@ def inv_frequencies(head_dim: int, theta: float, scaling=None):
 class Rotary(PositionEncoding):
     graph_safe = True
 
-    def __init__(self, env, head_dim: int, theta: float, scaling=None, pairing: str = "half"):
-        if head_dim % 2:
-            raise ValueError(f"rotary: head size {head_dim} must be even")
+    def __init__(self, env, head_dim: int, theta: float, scaling=None, pairing: str = "half", rotary_dim=None):
+        """``rotary_dim``: only the first so many elements of a head rotate, with the frequencies of
+        a head of that size; the rest pass through (default: the whole head)."""
+        rot = head_dim if rotary_dim is None else int(rotary_dim)
+        if head_dim % 2 or rot % 2 or not 0 < rot <= head_dim:
+            raise ValueError(f"rotary: head size {head_dim} and rotating part {rot} must be even, the part within the head")
         if pairing not in ("half", "adjacent"):
             raise ValueError(f"rotary: pairing {pairing!r}")
         if scaling is not None and scaling.get("rope_type", "llama3") != "llama3":
             raise ValueError(f"rotary: scaling of type {scaling.get('rope_type')!r} is not known")
         self.adjacent = pairing == "adjacent"
-        self.inv_freq = torch.tensor(inv_frequencies(head_dim, theta, scaling), dtype=torch.float64) \
+        self.rotary_dim = rot
+        self.inv_freq = torch.tensor(inv_frequencies(rot, theta, scaling), dtype=torch.float64) \
             .to(torch.float32).to(env.device)
 
     def kernel_args(self):
-        return {"use_rope": True, "inv_freq": self.inv_freq, "adjacent": self.adjacent}
+        return {"use_rope": True, "inv_freq": self.inv_freq, "adjacent": self.adjacent, "rotary_dim": self.rotary_dim}
 
 
 @register("position", "none")

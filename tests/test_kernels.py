@@ -117,6 +117,50 @@ def test_rope_kvwrite(dtype, H, G, hd, adjacent, norm, temp, T):
                 assert float(kp[p, :, o].abs().sum()) == 0 and float(vp[p, :, :, o].abs().sum()) == 0
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,G,hd,rot,adjacent,weighted,first", [
+    (4, 2, 64, 32, False, True, True),      # half of the head rotates; weighted norm before the rotation
+    (3, 1, 48, 16, True, True, False),      # adjacent pairs, a third rotates; weighted norm after it
+    (6, 2, 128, 128, False, True, True),    # the whole head, weighted, norm first
+    (2, 2, 32, 8, False, False, True),      # weightless norm first: the same numbers as norm after (rotation keeps lengths)
+])
+def test_rope_kvwrite_with_part_of_the_head_rotating_and_a_weighted_norm_before_or_after(dtype, H, G, hd, rot, adjacent, weighted, first):
+    T, ps, n_pages = 37, 8, 6
+    qkv = rnd(T, (H + 2 * G) * hd, dtype=dtype, seed=3)
+    pos = ((torch.arange(T) * 7) % 50).to(torch.int32).to(DEV)
+    slots = torch.randperm(n_pages * ps, generator=torch.Generator().manual_seed(1))[:T].to(torch.int32).to(DEV)
+    inv = plain.rope_inv_freq(rot, 10000.0, None).to(torch.float32).to(DEV)
+    wq, wk = (rnd(hd, seed=5) * 0.3 + 1.0, rnd(hd, seed=6) * 0.3 + 1.0) if weighted else (None, None)
+    q = torch.empty(T, H * hd, dtype=dtype, device=DEV)
+    kp = torch.zeros(n_pages, G, ps, hd, dtype=dtype, device=DEV)
+    vp = torch.zeros(n_pages, G, hd, ps, dtype=dtype, device=DEV)
+    ops().rope_kvwrite(qkv, q, kp, vp, pos, slots, inv, H, G, hd, ps, use_rope=True, adjacent=adjacent, use_norm=True,
+                       norm_eps=1e-5, use_temp=False, floor_scale=1, attn_scale=0.0, rotary_dim=rot,
+                       norm_weight_q=wq, norm_weight_k=wk, norm_first=first)
+    x = qkv.double().cpu()
+    qq, kk = x[:, :H * hd].view(T, H, hd), x[:, H * hd:(H + G) * hd].view(T, G, hd)
+    pc, pairing = pos.cpu(), "adjacent" if adjacent else "half"
+
+    def rotate(v):        # the first `rot` elements as a head of that size, the rest untouched
+        out = v.clone()
+        out[..., :rot] = plain.apply_rope(v[..., :rot], pc, inv.double().cpu(), pairing)
+        return out
+
+    def norm(v, w):
+        y = plain.rms_norm(v, None, 1e-5)
+        return y if w is None else y * w.double().cpu()
+    want_q, want_k = (rotate(norm(qq, wq)), rotate(norm(kk, wk))) if first else (norm(rotate(qq), wq), norm(rotate(kk), wk))
+    tol = tol_for(dtype, want_q) * (4 if dtype == torch.float32 else 1.5)
+    assert (q.double().cpu().view(T, H, hd) - want_q).abs().max() < tol
+    for t in range(T):
+        page, off = int(slots[t]) // ps, int(slots[t]) % ps
+        assert (kp[page, :, off].double().cpu() - want_k[t]).abs().max() < tol
+    # a wrong order of norm and rotation shows where the weights are not all alike
+    if weighted:
+        other_q = norm(rotate(qq), wq) if first else rotate(norm(qq, wq))
+        assert (other_q - want_q).abs().max() > 20 * tol
+
+
 def test_rope_kvwrite_refuses_odd_sizes():
     from spite_amd.csrc.hipops import KernelError
     z = torch.zeros(1, 3 * 15, device=DEV)

@@ -372,3 +372,52 @@ def test_other_ends_of_a_model_an_embedding_with_a_scale_and_a_head_with_a_cap_a
         err = max(abs(got[("x", i)] - ref[i]).max() for i in range(T))
         assert err < 1e-4, err
     assert abs(ref).max() > 1.5            # the cap is felt
+
+
+def test_attention_with_a_weighted_head_norm_before_a_rotation_of_part_of_the_head():
+    """What other architectures' attention needs beside Llama 4's: the head norm with weights, placed
+    before the rotation, and a rotation of the head's first elements only - options of the built-in
+    mixer and position encoding, chosen by the spec."""
+    from spite_amd import Engine
+    from spite_amd.parts import PartSpec, BlockSpec, LayerCall, ModelSpec
+    import plain_llama4 as plain
+    rot = 4
+    rms = lambda name: PartSpec("rms", {"width": D, "eps": 1e-5}, {"weight": name})
+    names = {k: f"b1.attn.{k}" for k in ("q_proj", "k_proj", "v_proj", "o_proj")}
+    names.update(q_norm="b1.attn.q_norm", k_norm="b1.attn.k_norm")
+    attn = PartSpec("attention", dict(hidden_size=D, n_heads=HEADS, n_kv_heads=KV, head_dim=HD, qk_norm=True, qk_norm_eps=1e-6,
+                                      qk_norm_weighted=True, qk_norm_first=True,
+                                      position=PartSpec("rotary", {"head_dim": HD, "theta": 100.0, "rotary_dim": rot})), names)
+    dense = PartSpec("dense_glu", {"hidden_size": D, "intermediate_size": 40},
+                     {k: f"b1.ffn.{k}" for k in ("gate_proj", "up_proj", "down_proj")})
+    sp = ModelSpec("ToyNormFirst", V, D, [BlockSpec("prenorm", rms("b1.n1"), attn, rms("b1.n2"), dense)], [LayerCall(0, 0)],
+                   rms("final"), "embed", "head")
+    t = {k: v for k, v in tensors(4).items() if k in ("embed", "head", "final") or k.startswith("b1.")}
+    g = torch.Generator().manual_seed(9)
+    t["b1.attn.q_norm"], t["b1.attn.k_norm"] = 1 + torch.randn(HD, generator=g) * 0.4, 1 + torch.randn(HD, generator=g) * 0.4
+    W = {k: v.double() for k, v in t.items()}
+    toks = H.random_tokens(V, 26, 8)
+    T, pos = len(toks), torch.arange(len(toks))
+    inv = plain.rope_inv_freq(rot, 100.0, None)
+
+    def rotate(x):
+        out = x.clone()
+        out[..., :rot] = plain.apply_rope(x[..., :rot], pos, inv)
+        return out
+    h = W["embed"][torch.tensor(toks)]
+    n = plain.rms_norm(h, W["b1.n1"], 1e-5)
+    q = rotate(plain.rms_norm((n @ W["b1.attn.q_proj"].T).view(T, HEADS, HD), W["b1.attn.q_norm"], 1e-6))
+    k = rotate(plain.rms_norm((n @ W["b1.attn.k_proj"].T).view(T, KV, HD), W["b1.attn.k_norm"], 1e-6))
+    v = (n @ W["b1.attn.v_proj"].T).view(T, KV, HD)
+    h = h + plain.attention(q, k, v, plain.visible_mask(pos, "full", 0)).reshape(T, HEADS * HD) @ W["b1.attn.o_proj"].T
+    h = h + plain.swiglu_mlp(plain.rms_norm(h, W["b1.n2"], 1e-5), W["b1.ffn.gate_proj"], W["b1.ffn.up_proj"], W["b1.ffn.down_proj"])
+    ref = (plain.rms_norm(h, W["final"], 1e-5) @ W["head"].T).float().numpy()
+    reqs = {"x": toks}
+    eng = Engine(spec=sp, tensors=t, dtype="float32", page_size=4, cache_tokens=64, max_requests=2)
+    for steps in (H.schedule_whole(reqs), H.schedule_tail_one_by_one(reqs, tail=9)):
+        got = H.collect(steps, H.run_trace_inprocess(eng, steps), V)
+        err = max(abs(got[("x", i)] - ref[i]).max() for i in range(T))
+        assert err < 1e-4, err
+    # the test has teeth: the other order of norm and rotation is another function
+    q2 = plain.rms_norm(rotate((n @ W["b1.attn.q_proj"].T).view(T, HEADS, HD)), W["b1.attn.q_norm"], 1e-6)
+    assert (q2 - q).abs().max() > 0.05
