@@ -377,7 +377,8 @@ extern "C" int spite_gemm_tiled_split(const void* X, int ldx, const void* W, voi
 // `shape`: 0 lets the library choose; 1 = 512 W rows x 128 slots a workgroup, 2 = 256 x 256,
 // 3 = 512 x 160 (for groups of a little over 128 rows, which would need a second tile of 128),
 // 4 and 5 = 512 x 64 with W asked for five half steps ahead (short prompts: the stream of W from
-// memory is the time; 4 reads W with non-temporal loads, 5 with plain ones).
+// memory is the time; 4 reads W with non-temporal loads, 5 with plain ones), 6 = 512 x 96 (plain
+// products only).
 extern "C" int spite_gemm_tiled(const void* X, int ldx, const void* W, long w_group_stride, void* Y, int y_dtype,
                                 int ldy, int M, int N, int K, const int* offsets, int n_groups, const int* a_rows,
                                 const float* a_scale, const int* y_rows, int glu, int shape, hipStream_t st) {
@@ -387,9 +388,26 @@ extern "C" int spite_gemm_tiled(const void* X, int ldx, const void* W, long w_gr
     SP_REQUIRE(((uintptr_t)X & 15) == 0 && ((uintptr_t)W & 15) == 0, "gemm_tiled: operands must be 16-byte aligned");
     SP_REQUIRE(y_dtype == SP_BF16 || y_dtype == SP_F32, "gemm_tiled: output dtype %d", y_dtype);
     SP_REQUIRE(!offsets || n_groups > 0, "gemm_tiled: grouped call without groups");
-    SP_REQUIRE(shape >= 0 && shape <= 5, "gemm_tiled: tile shape %d", shape);
+    SP_REQUIRE(shape >= 0 && shape <= 6, "gemm_tiled: tile shape %d", shape);
     if (M == 0) return 0;
-    if (shape == 0) shape = 1;          // measured the faster one at every shape of Llama 4 Scout
+    if (shape == 0) {
+        // Tiles come in whole numbers per CU: a plain product whose 128-row tiles leave many of the 256
+        // CUs without one (2,048 x 5,120: 160 tiles) takes 96-row tiles when those need no further round
+        // (220 tiles).  A tile's time was measured as 38 + 8.5 us per 16 rows at K = 5,120; the sum over
+        // k runs in the same order in both, so a row's result does not depend on the choice.
+        shape = 1;
+        if (!offsets && !glu) {
+            const long cols = (N + 511) / 512;
+            const long rounds8 = (((M + 127) / 128) * cols + 255) / 256, rounds6 = (((M + 95) / 96) * cols + 255) / 256;
+            if (rounds6 * (38 + 8.5 * 6) < rounds8 * (38 + 8.5 * 8)) shape = 6;
+        }
+    }
+    if (shape == 6) {
+        SP_REQUIRE(!offsets && !glu, "gemm_tiled: the 96-row tile is for plain products");
+        return y_dtype == SP_BF16
+            ? launch_tiled_kernel<8, 1, 6, false, bf16, false>(X, ldx, W, w_group_stride, Y, ldy, M, N, K, nullptr, 1, a_rows, a_scale, y_rows, 1, 0, st)
+            : launch_tiled_kernel<8, 1, 6, false, float, false>(X, ldx, W, w_group_stride, Y, ldy, M, N, K, nullptr, 1, a_rows, a_scale, y_rows, 1, 0, st);
+    }
     if (shape == 1)
         return launch_tiled<8, 1, 8>(X, ldx, W, w_group_stride, Y, y_dtype, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu, st);
     if (shape == 4 || shape == 5) {

@@ -266,6 +266,30 @@ def test_gemm_tiled(M, N, K, out_dtype, glu, grouped, shape):
     run_gemm(fn, torch.bfloat16, out_dtype, M, N, K, glu, grouped, shape=shape)
 
 
+@pytest.mark.parametrize("M,N,K", [(200, 304, 256), (97, 528, 192), (520, 1040, 128), (2048, 1024, 128)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_gemm_tiled_with_rows_in_tiles_of_96(M, N, K, out_dtype):
+    """The tile that a plain product takes where its 128-row tiles would leave CUs without one: the
+    same bits as the 128-row tile (the sum over k runs in the same order), also as the library's own
+    choice, which takes it at the last of these sizes (16 x 2 tiles of 128 rows, 22 x 2 of 96)."""
+    def fn(shape):
+        def run(a, w, y, *args, **kw):
+            ops().gemm_tiled(a, ops().operand_order(w), y, *args, shape=shape, **kw)
+        return run
+    run_gemm(fn(6), torch.bfloat16, out_dtype, M, N, K)
+    a, w = rnd(M, K, dtype=torch.bfloat16, seed=1), ops().operand_order(rnd(N, K, dtype=torch.bfloat16, seed=2))
+    ys = []
+    for shape in (1, 6, 0):
+        y = torch.empty(M, N, dtype=out_dtype, device=DEV)
+        ops().gemm_tiled(a, w, y, M, N, K, shape=shape)
+        ys.append(y)
+    assert torch.equal(ys[0], ys[1]) and torch.equal(ys[0], ys[2])
+    from spite_amd.csrc.hipops import KernelError
+    with pytest.raises(KernelError, match="plain products"):
+        ops().gemm_tiled(a[:8, :64].contiguous(), ops().operand_order(rnd(64, 64, dtype=torch.bfloat16)),
+                         torch.empty(8, 32, dtype=out_dtype, device=DEV), 8, 32, 64, glu=True, shape=6)
+
+
 @pytest.mark.parametrize("M,groups", [(40, 150), (300, 150), (9, 64), (70, 65), (500, 129)])
 @pytest.mark.parametrize("glu", [False, True])
 def test_gemm_over_many_groups(M, groups, glu):
