@@ -37,6 +37,13 @@ class Workspace:
             self.generation += 1
         self._off = 0
 
+    def mark(self) -> int:
+        """Where the next ``take`` starts; ``rewind`` goes back there (within one generation)."""
+        return self._off
+
+    def rewind(self, mark: int) -> None:
+        self._off = mark
+
     def take(self, shape, dtype) -> torch.Tensor:
         n = 1
         for s in shape:

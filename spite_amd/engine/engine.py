@@ -174,8 +174,8 @@ class Engine:
         self._pin_event = None
         self._meta_dev = None
         self.steps_run = 0
-        self.use_graphs = bool(graphs) and self.model.graph_safe
-        self._graphs: Dict[tuple, object] = {}     # shape of a decode step -> (graph, logits) or "seen"
+        self.use_graphs = bool(graphs) and any(safe for _, _, safe in self.model.graph_segments())
+        self._graphs: Dict[tuple, object] = {}     # shape of a decode step -> (segments, state), "seen" once, or "eager" for good
         self._graph_stamp = None
         self.graph_replays = 0
 
@@ -257,14 +257,14 @@ class Engine:
         if (self.use_graphs and trace is None and meta.ctx.decode_only and meta.ctx.n_out == meta.ctx.n_seqs
                 and all(tuple(e.want) == (0,) for e in entries)):
             key = (meta.ctx.n_seqs, meta.widths)
-            logits = self._replay(key)
+            logits = self._replay(key, meta)
         if logits is None:
             self._step_ws.reset()
             if key is not None and self._graphs.get(key) == "seen":
                 logits = self._capture(key, meta)
             else:
                 logits = self.model.forward(meta.ctx, self.cache, meta, self._arenas, self._step_ws)
-                if key is not None:
+                if key is not None and key not in self._graphs:
                     self._graphs[key] = "seen"
                 # this step may have grown a workspace (a first decode step of a larger shape
                 # does): graphs captured before point into memory that the merge frees
@@ -287,44 +287,84 @@ class Engine:
         stamp = self._stamp()
         if stamp == self._graph_stamp:
             return False
-        self._graphs = {k: v for k, v in self._graphs.items() if v == "seen"}
+        self._graphs = {k: v for k, v in self._graphs.items() if isinstance(v, str)}
         self._graph_stamp = stamp
         return True
 
-    def _replay(self, key):
+    # A captured step is a row of segments of the model's units: graphs over the runs of units
+    # that can be captured, and between them the units that cannot (a part that reads the step's
+    # metadata on the host), which run eagerly in every step on the buffers the graphs know.
+    def _run_eager(self, lo, hi, state, meta):
+        return self.model.run_units(lo, hi, state, meta.ctx, self.cache, meta, self._arenas, self._step_ws)
+
+    @staticmethod
+    def _addresses(state):
+        return tuple((k, tuple(t.data_ptr() for t in (v if isinstance(v, tuple) else (v,)) if isinstance(t, torch.Tensor)))
+                     for k, v in sorted(state.items()) if k != "logits")
+
+    def _replay(self, key, meta):
         if self._drop_stale_graphs():
             return None
         hit = self._graphs.get(key)
-        if hit is None or hit == "seen":
+        if hit is None or isinstance(hit, str):
             return None
-        graph, logits = hit
-        graph.replay()
+        segments, state = hit
+        for n, (lo, hi, graph, after) in enumerate(segments):
+            if graph is not None:
+                graph.replay()
+                continue
+            # the eager units of this step: the same buffers as in the captured step, or the rest
+            # of the step runs eagerly too and the graphs are dropped
+            live = dict(after["before"])
+            for ws, mark in zip((*self._arenas, self._step_ws), after["marks"]):
+                ws.rewind(mark)
+            self._run_eager(lo, hi, live, meta)
+            if self._stamp() != self._graph_stamp:
+                self._graphs.pop(key, None)            # a buffer grew: captured anew when the shape comes up again
+                self._drop_stale_graphs()
+                return self._run_eager(hi, self.model.n_units(), live, meta)["logits"]
+            if self._addresses(live) != after["addresses"]:
+                # a part hands on memory of its own instead of the step's workspace: what follows
+                # it cannot be replayed, so steps of this shape run eagerly from now on
+                self._graphs[key] = "eager"
+                return self._run_eager(hi, self.model.n_units(), live, meta)["logits"]
         self.graph_replays += 1
-        return logits
+        return state["logits"]
 
     def _capture(self, key, meta):
         for ws in self._arenas:
             ws.reset()                     # merge what the warm-up step added, outside the capture
         self._drop_stale_graphs()          # the merge has freed what older graphs point into
-        graph = torch.cuda.CUDAGraph()
-        try:
-            with torch.cuda.graph(graph):
-                logits = self.model.forward(meta.ctx, self.cache, meta, self._arenas, self._step_ws)
-        except Exception:
-            self._graphs.pop(key, None)
-            self.use_graphs = False        # fall back to eager steps for good, loudly
-            import warnings
-            warnings.warn("capturing the decode step in a HIP graph failed; steps run eagerly from now on")
-            self._step_ws.reset()
-            return self.model.forward(meta.ctx, self.cache, meta, self._arenas, self._step_ws)
-        if self._drop_stale_graphs():      # cannot happen (a workspace refuses to grow under capture)
-            self._graphs.pop(key, None)
-            self._step_ws.reset()
-            return self.model.forward(meta.ctx, self.cache, meta, self._arenas, self._step_ws)
-        graph.replay()                     # the capture itself computed nothing
-        self._graphs[key] = (graph, logits)
+        segments, state = [], {}
+        for lo, hi, safe in self.model.graph_segments():
+            if not safe:
+                before, marks = dict(state), tuple(ws.mark() for ws in (*self._arenas, self._step_ws))
+                self._run_eager(lo, hi, state, meta)
+                segments.append((lo, hi, None, {"before": before, "marks": marks, "addresses": self._addresses(state)}))
+                continue
+            graph = torch.cuda.CUDAGraph()
+            try:
+                with torch.cuda.graph(graph):
+                    self._run_eager(lo, hi, state, meta)
+            except Exception:
+                # nothing of this segment has run yet (a capture computes nothing): the rest of the
+                # step runs eagerly, and so does every later step, loudly
+                self._graphs.pop(key, None)
+                self.use_graphs = False
+                import warnings
+                warnings.warn("capturing the decode step in a HIP graph failed; steps run eagerly from now on")
+                if lo == 0:
+                    self._step_ws.reset()
+                    state = {}
+                return self._run_eager(lo, self.model.n_units(), state, meta)["logits"]
+            if self._drop_stale_graphs():  # cannot happen (a workspace refuses to grow under capture)
+                self._graphs.pop(key, None)
+                return self._run_eager(lo, self.model.n_units(), state, meta)["logits"]
+            graph.replay()                 # the capture itself computed nothing
+            segments.append((lo, hi, graph, None))
+        self._graphs[key] = (segments, state)
         self.graph_replays += 1
-        return logits
+        return state["logits"]
 
     def commit(self, entries: Sequence[StepEntry]) -> None:
         for e in entries:

@@ -39,8 +39,8 @@ class Model:
             if not call.write and (call.cache not in writers or writers[call.cache] > i):
                 raise ValueError(f"layer call {i} reads cache {call.cache} before any call has written it")
         self._writers = writers
-        self.graph_safe = all(b.graph_safe for b in self.blocks) and self.final_norm.graph_safe \
-            and self.embedding.graph_safe and self.head.graph_safe
+        self._units = self._build_units()
+        self.graph_safe = all(u[1] for u in self._units)
         self.step_arrays = tuple(sorted({a for b in self.blocks for a in b.step_arrays}))
 
     # ------------------------------------------------------------------ tensors
@@ -76,25 +76,61 @@ class Model:
         return needs
 
     # ------------------------------------------------------------------ one step
+    # A step is a row of units: the embedding, every layer call, and the tail (final norm and
+    # head).  ``forward`` runs them all; the engine's graphs run them in segments, so that a part
+    # that cannot be captured costs an eager call of its own unit and nothing else.
+    def _build_units(self):
+        units = [("embed", self.embedding.graph_safe, None, None)]
+        for i, call in enumerate(self.spec.order):
+            for j, (safe, fn) in enumerate(self.blocks[call.block].stages()):
+                units.append(("stage", bool(safe), i, (j, fn)))
+        units.append(("tail", self.final_norm.graph_safe and self.head.graph_safe, None, None))
+        return units
+
+    def n_units(self) -> int:
+        return len(self._units)
+
+    def graph_segments(self) -> List[Tuple[int, int, bool]]:
+        """Maximal runs of units ``(first, end, safe)`` that can (or cannot) be captured."""
+        segs, lo, units = [], 0, self._units
+        for u in range(1, len(units) + 1):
+            if u == len(units) or units[u][1] != units[lo][1]:
+                segs.append((lo, u, units[lo][1]))
+                lo = u
+        return segs
+
+    def run_units(self, lo: int, hi: int, state: dict, ctx: StepContext, cache, meta, arenas, step_ws: Workspace) -> dict:
+        """Runs units ``lo .. hi-1``.  ``state`` carries the residual stream ``h``, the increments
+        that the next norm has to add (``pending``), what a block's stages hand each other and,
+        after the tail, ``logits``."""
+        n, d = len(self.spec.order), self.spec.hidden_size
+        for u in range(lo, hi):
+            kind, _, i, stage = self._units[u]
+            if kind == "embed":
+                state["h"] = step_ws.take((ctx.T, d), torch.float32)
+                state["pending"] = ()
+                ctx.ws = arenas[0]
+                self.embedding.forward(ctx.token_ids, state["h"], ctx)
+            elif kind == "stage":
+                ctx.ws = arenas[i % 2]
+                if stage[0] == 0:
+                    ctx.ws.reset()
+                stage[1](state, ctx, meta.layer_cache(cache, self.spec.order[i]))
+            else:
+                ctx.ws = arenas[n % 2]
+                ctx.ws.reset()
+                if ctx.n_out == 0:
+                    state["logits"] = torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.env.device)
+                    continue
+                pending = state["pending"]
+                rows = ctx.ws.take((ctx.n_out, d), self.env.dtype)
+                self.final_norm.forward(state["h"], rows, d1=pending[0] if len(pending) > 0 else None,
+                                        d2=pending[1] if len(pending) > 1 else None, rows=ctx.logit_rows, write_h=False)
+                state["logits"] = step_ws.take((ctx.n_out, self.spec.vocab_size), torch.float32)
+                self.head.forward(rows, state["logits"], ctx)
+        return state
+
     def forward(self, ctx: StepContext, cache, meta, arenas, step_ws: Workspace) -> torch.Tensor:
         """Runs the tokens of the step through every layer call; returns fp32 logits
         ``[n_out, V]`` at ``ctx.logit_rows``."""
-        T, d = ctx.T, self.spec.hidden_size
-        h = step_ws.take((T, d), torch.float32)
-        ctx.ws = arenas[0]
-        self.embedding.forward(ctx.token_ids, h, ctx)
-        pending = ()
-        for i, call in enumerate(self.spec.order):
-            ctx.ws = arenas[i % 2]
-            ctx.ws.reset()
-            pending = self.blocks[call.block].forward(h, pending, ctx, meta.layer_cache(cache, call))
-        ctx.ws = arenas[len(self.spec.order) % 2]
-        ctx.ws.reset()
-        if ctx.n_out == 0:
-            return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.env.device)
-        n = ctx.ws.take((ctx.n_out, d), self.env.dtype)
-        self.final_norm.forward(h, n, d1=pending[0] if len(pending) > 0 else None,
-                                d2=pending[1] if len(pending) > 1 else None, rows=ctx.logit_rows, write_h=False)
-        logits = step_ws.take((ctx.n_out, self.spec.vocab_size), torch.float32)
-        self.head.forward(n, logits, ctx)
-        return logits
+        return self.run_units(0, self.n_units(), {}, ctx, cache, meta, arenas, step_ws)["logits"]

@@ -182,6 +182,16 @@ class Block(Part):
         increments not yet added to h.  Returns the new pending increments."""
         raise NotImplementedError
 
+    def stages(self):
+        """The block's forward as a row of ``(graph_safe, fn(state, ctx, cache))``, cut where a part
+        that cannot be captured in a graph begins or ends; run in order they are ``forward``.
+        ``state["h"]`` and ``state["pending"]`` are forward's arguments and result; a stage may
+        leave what the next one needs under keys of its own.  The engine's graphs hold the safe
+        stages; the others run eagerly between them.  Default: the whole block as one stage."""
+        def whole(state, ctx, cache):
+            state["pending"] = self.forward(state["h"], state["pending"], ctx, cache)
+        return [(self.graph_safe, whole)]
+
 
 # ----------------------------------------------------------------------------- derived step metadata
 _STEP_ARRAYS: Dict[str, Callable] = {}

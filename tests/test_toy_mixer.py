@@ -182,3 +182,89 @@ def test_the_toy_mixer_is_served_by_generate_with_preemption_on_a_tiny_pool():
     for p, g in zip(prompts, got):
         assert g == plain_generate(p, 7)
     eng.cache.check()
+
+
+def test_graphs_hold_what_can_be_captured_around_a_mixer_that_cannot_be():
+    """The toy mixer walks requests on the host, so it cannot be captured; the engine's graphs
+    hold the units around it (embedding and first norm | feed-forward up to the next toy mixer's
+    norm | the rest) and the mixer runs eagerly between them, on the buffers the graphs know.
+    Same logits as eager steps, bit for bit, while requests come, go and take used slots."""
+    from spite_amd import Engine, StepEntry
+    define_parts()
+    t = tensors(2)
+    engines = [Engine(spec=spec("full", 0), tensors=t, dtype="float32", page_size=4, cache_tokens=400, max_requests=4, graphs=g)
+               for g in (True, False)]
+    assert engines[0].use_graphs and not engines[0].model.graph_safe
+    kinds = [safe for _, _, safe in engines[0].model.graph_segments()]
+    assert kinds == [True, False, True, False, True]
+    prompts = [H.random_tokens(V, n, 70 + n) for n in (5, 9, 3, 7)]
+    outs = []
+    for eng in engines:
+        rows, slots, last = [], {}, {}
+        for i in (0, 1, 2):
+            slots[i] = eng.admit()
+            last[i] = int(eng.step([StepEntry(slots[i], prompts[i], [len(prompts[i]) - 1])])[0].argmax())
+        for step in range(40):
+            if step == 12:                   # one request ends, another takes its slot and its state rows
+                eng.release(slots.pop(1))
+                slots[3] = eng.admit()
+                last[3] = int(eng.step([StepEntry(slots[3], prompts[3], [len(prompts[3]) - 1])])[0].argmax())
+                del last[1]
+            ids = sorted(slots)
+            logits = eng.step([StepEntry(slots[i], [last[i]], [0]) for i in ids]).cpu()
+            rows.append(logits.clone())
+            for j, i in enumerate(ids):
+                last[i] = int(logits[j].argmax())
+        outs.append(rows)
+    assert engines[0].graph_replays >= 30 and engines[1].graph_replays == 0
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    # against the plain model: the first request's tokens, all forty of them
+    toks = list(prompts[0])
+    for step in range(40):
+        row = plain_toy(t, toks, "full", 0)[-1] if step == 0 else ref
+        toks.append(int(row.argmax()))
+        ref = plain_toy(t, toks, "full", 0)[-1]
+        assert abs(outs[0][step][0].numpy() - ref).max() < 1e-4, step
+
+
+def test_a_part_that_hands_on_memory_of_its_own_keeps_its_steps_eager():
+    """A mixer that returns a tensor of torch's instead of one from the step's workspace: what
+    follows it cannot be replayed from a graph.  The engine notices at the first replay, finishes
+    that step eagerly and runs steps of that shape eagerly from then on; the logits are right."""
+    from spite_amd import Engine, StepEntry
+    from spite_amd.parts import Mixer, ParamSpec, CacheNeed, register, PartSpec, BlockSpec, LayerCall, ModelSpec
+
+    @register("mixer", "toy_own_memory")
+    class OwnMemory(Mixer):
+        def __init__(self, env, width):
+            self.width, self.w = width, None
+
+        def params(self):
+            return {"proj": ParamSpec((self.width, self.width))}
+
+        def load(self, tensors):
+            self.w = tensors["proj"]
+
+        def cache_need(self):
+            return CacheNeed()
+
+        def forward(self, x, ctx, cache):
+            self.keep = getattr(self, "keep", []) + [torch.empty(64, device=x.device)]     # the allocator moves on
+            return x.float() @ self.w.float().T
+
+    norm = lambda name: PartSpec("rms", {"width": D, "eps": 1e-5}, {"weight": name})
+    ffn = PartSpec("dense_glu", {"hidden_size": D, "intermediate_size": 48}, {k: f"b0.ffn.{k}" for k in ("gate_proj", "up_proj", "down_proj")})
+    sp = ModelSpec("ToyOwn", V, D, [BlockSpec("prenorm", norm("b0.n1"), PartSpec("toy_own_memory", {"width": D}, {"proj": "b0.mix"}),
+                                              norm("b0.n2"), ffn)], [LayerCall(0, 0)], norm("final"), "embed", "head")
+    t = {k: v for k, v in tensors(3).items() if k in ("embed", "head", "final") or k.startswith("b0.")}
+    outs = []
+    for graphs in (True, False):
+        eng = Engine(spec=sp, tensors=t, dtype="float32", page_size=4, cache_tokens=64, max_requests=2, graphs=graphs)
+        s = eng.admit()
+        eng.step([StepEntry(s, [1, 2, 3], [])])
+        outs.append([eng.step([StepEntry(s, [4 + i], [0])]).cpu().clone() for i in range(8)])
+        if graphs:
+            assert "eager" in eng._graphs.values() and eng.graph_replays <= 1
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)

@@ -174,7 +174,7 @@ def test_other_norms_position_encodings_and_routed_feed_forwards_are_built_and_s
         and "toy_top2_softmax" in registered("ffn")
     t = tensors()
     eng = Engine(spec=spec(), tensors=t, dtype="float32", page_size=4, cache_tokens=96, max_requests=3)
-    assert not eng.use_graphs                     # the toy parts do not claim to be safe to capture
+    assert not eng.model.graph_safe               # the toy parts do not claim to be safe to capture; what is, is captured
     assert eng.cache.n_groups() == 2              # a full group and a window group
     reqs = {"x": H.random_tokens(V, 23, 1), "y": H.random_tokens(V, 9, 2), "z": H.random_tokens(V, 15, 3)}
     ref = {(rid, i): row for rid, toks in reqs.items() for i, row in enumerate(plain_toy(t, toks))}
