@@ -16,10 +16,10 @@ from typing import Dict, List, Optional, Sequence
 import numpy as np
 import torch
 
-from ..csrc import hostlib, hipops
+from ..csrc import build, hostlib, hipops
 from ..parts.base import CacheNeed
 
-_KINDS = {"full": 0, "chunk": 1, "window": 2}
+_KINDS = build.visibility_codes()     # "full", "chunk", "window": name -> code
 
 
 class CacheError(RuntimeError):

@@ -58,7 +58,19 @@ def _sources(kind: str):
     folder = os.path.join(_HERE, sub)
     srcs = sorted(os.path.join(folder, f) for f in os.listdir(folder) if f.endswith(ext))
     deps = sorted(os.path.join(folder, f) for f in os.listdir(folder) if f.endswith(".h"))
+    deps.append(os.path.join(_HERE, "visibility.h"))          # shared by both libraries
     return srcs, deps
+
+
+def visibility_codes() -> dict:
+    """Name -> code of the rules that say which keys a query may read, as ``visibility.h``
+    lists them (the header both libraries are built from is the one place that defines them)."""
+    import re
+    with open(os.path.join(_HERE, "visibility.h")) as f:
+        m = re.search(r'#define\s+SP_VIS_NAMES\s+"([^"]*)"', f.read())
+    if not m:
+        raise BuildError("visibility.h does not list the rules' names")
+    return {name: i for i, name in enumerate(m.group(1).split(","))}
 
 
 def _find_hipcc() -> str:

@@ -229,7 +229,7 @@ extern "C" int spite_attn_decode(const void* q, const void* k_pages, const void*
     SP_REQUIRE(hd == 64 || hd == 128, "attn_decode: head size %d (this kernel has 64 and 128)", hd);
     SP_REQUIRE(page_size > 0 && page_size % 32 == 0, "attn_decode: page size %d must be a multiple of 32", page_size);
     SP_REQUIRE(max_blocks > 0 && n_splits >= 1 && n_splits <= 256, "attn_decode: bad table width, or %d splits (at most 256)", n_splits);
-    SP_REQUIRE(vis == SP_VIS_FULL || span > 0, "attn_decode: chunk or window of %d", span);
+    SP_REQUIRE(vis >= 0 && vis < SP_VIS_COUNT && (!sp_vis_has_span(vis) || span > 0), "attn_decode: chunk or window of %d", span);
     SP_REQUIRE(G <= 65535 && T <= 65535, "attn_decode: too many heads or tokens for one launch");
     if (T == 0) return 0;
     const float sl = scale * 1.4426950408889634f;

@@ -93,7 +93,7 @@ extern "C" int spite_attn_generic(const void* q, const void* k_pages, const void
     SP_REQUIRE(T >= 0 && H > 0 && G > 0 && H % G == 0, "attention: %d query heads over %d kv heads", H, G);
     SP_REQUIRE(hd > 0 && hd <= 64 * ATT_MAX_D, "attention: head size %d, at most %d", hd, 64 * ATT_MAX_D);
     SP_REQUIRE(page_size > 0 && max_blocks > 0, "attention: bad page size %d or table width %d", page_size, max_blocks);
-    SP_REQUIRE(vis == SP_VIS_FULL || span > 0, "attention: chunk or window of %d", span);
+    SP_REQUIRE(vis >= 0 && vis < SP_VIS_COUNT && (!sp_vis_has_span(vis) || span > 0), "attention: chunk or window of %d", span);
     SP_REQUIRE(H <= 65535, "attention: too many heads");
     SP_REQUIRE(!kv_tiled || (dtype == SP_BF16 && hd % 32 == 0 && page_size % 32 == 0),
                "attention: pages in operand order are bfloat16 with head size %d and page size %d multiples of 32", hd, page_size);

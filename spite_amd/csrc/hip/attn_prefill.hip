@@ -329,7 +329,7 @@ extern "C" int spite_attn_prefill(const void* q, const void* k_pages, const void
     SP_REQUIRE(hd == 64 || hd == 128, "attn_prefill: head size %d (this kernel has 64 and 128)", hd);
     SP_REQUIRE(page_size > 0 && page_size % 32 == 0, "attn_prefill: page size %d must be a multiple of 32", page_size);
     SP_REQUIRE(max_blocks > 0, "attn_prefill: bad table width");
-    SP_REQUIRE(vis == SP_VIS_FULL || span > 0, "attn_prefill: chunk or window of %d", span);
+    SP_REQUIRE(vis >= 0 && vis < SP_VIS_COUNT && (!sp_vis_has_span(vis) || span > 0), "attn_prefill: chunk or window of %d", span);
     SP_REQUIRE(G <= 65535, "attn_prefill: too many kv heads for one launch");
     SP_REQUIRE(key_split >= 0 && key_split <= 2, "attn_prefill: key split %d", key_split);
     long tiles[3] = {0, 0, 0};

@@ -13,8 +13,9 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 enum { SP_F32 = 0, SP_BF16 = 1 };
-// Which keys a query may read besides the causal rule j <= p.
-enum { SP_VIS_FULL = 0, SP_VIS_CHUNK = 1, SP_VIS_WINDOW = 2 };
+// Which keys a query may read besides the causal rule j <= p: shared with the cache manager.
+#define SP_VIS_FN __device__ __host__ __forceinline__
+#include "../visibility.h"
 
 #define SP_WAVE 64
 
@@ -25,12 +26,6 @@ int sp_fail(const char* fmt, ...);
 #define SP_LAUNCH_CHECK(name) do { hipError_t e_ = hipGetLastError(); \
     if (e_ != hipSuccess) return sp_fail("%s: launch failed: %s", name, hipGetErrorString(e_)); } while (0)
 
-// First position a query at p may read (the last is p itself).
-__device__ __forceinline__ int sp_first_visible(int p, int vis, int span) {
-    if (vis == SP_VIS_CHUNK) return (p / span) * span;
-    if (vis == SP_VIS_WINDOW) return p - span + 1 > 0 ? p - span + 1 : 0;
-    return 0;
-}
 
 // ---- layouts of one kv head's part of a cache page.
 // Row-major: keys [page_size][hd], values transposed [hd][page_size].

@@ -16,7 +16,7 @@ import torch
 from . import build
 
 F32, BF16 = 0, 1
-VIS = {"full": 0, "chunk": 1, "window": 2}
+VIS = build.visibility_codes()      # "full", "chunk", "window": name -> code
 
 
 class KernelError(RuntimeError):

@@ -11,8 +11,8 @@ CacheManager::CacheManager(int page_size, int max_requests, const std::vector<Gr
     if (max_requests < 1) throw std::invalid_argument("max_requests must be >= 1");
     for (const auto& g : groups_) {
         if (g.n_pages < 1) throw std::invalid_argument("every group needs at least one page");
-        if (g.kind != VIS_FULL && g.span < 1) throw std::invalid_argument("chunk or window must be >= 1");
-        if (g.kind < VIS_FULL || g.kind > VIS_WINDOW) throw std::invalid_argument("unknown visibility");
+        if (g.kind < 0 || g.kind >= SP_VIS_COUNT) throw std::invalid_argument("unknown visibility");
+        if (sp_vis_has_span(g.kind) && g.span < 1) throw std::invalid_argument("chunk or window must be >= 1");
     }
     free_.resize(groups_.size());
     for (size_t g = 0; g < groups_.size(); ++g) {
@@ -128,16 +128,16 @@ int CacheManager::release(int slot) {
 
 int64_t CacheManager::peak_pages(int64_t total, int64_t portion, int g) const {
     const int64_t ps = page_size_;
-    if (groups_[g].kind == VIS_FULL || portion < 1) return (total + ps - 1) / ps;
-    // A portion of n positions that starts at c reads from first_visible(c), at most span-1
+    const int64_t back = sp_vis_lookback(groups_[g].kind, groups_[g].span);
+    if (back < 0 || portion < 1) return (total + ps - 1) / ps;
+    // A portion of n positions that starts at c reads from first_visible(c), at most `back`
     // positions before c.  Portions start anywhere (the budget cuts them), so take the worst
     // alignment; chunks that are whole pages start on a page.
     const int64_t all = (total + ps - 1) / ps;
     const int64_t n = std::min(portion, total);
-    const int64_t span = groups_[g].span;
     int64_t worst;
-    if (groups_[g].kind == VIS_CHUNK && span % ps == 0) worst = (span - 1 + n + ps - 1) / ps;
-    else worst = (span + n - 2) / ps + 2;
+    if (groups_[g].kind == SP_VIS_CHUNK && groups_[g].span % ps == 0) worst = (back + n + ps - 1) / ps;
+    else worst = (back + n - 1) / ps + 2;
     return std::min(all, worst);
 }
 

@@ -17,9 +17,11 @@
 #include <string>
 #include <vector>
 
+#define SP_VIS_FN inline
+#include "../visibility.h"
+
 namespace spite {
 
-enum Visibility { VIS_FULL = 0, VIS_CHUNK = 1, VIS_WINDOW = 2 };
 
 struct GroupSpec {
     int kind;      // Visibility
@@ -27,12 +29,8 @@ struct GroupSpec {
     int n_pages;   // pool size
 };
 
-// First position that a query at position p may read.
-inline int64_t first_visible(int64_t p, int kind, int span) {
-    if (kind == VIS_CHUNK) return (p / span) * span;
-    if (kind == VIS_WINDOW) return p - span + 1 > 0 ? p - span + 1 : 0;
-    return 0;
-}
+// First position that a query at position p may read: the rule shared with the attention kernels.
+inline int64_t first_visible(int64_t p, int kind, int span) { return sp_first_visible<int64_t>(p, kind, span); }
 
 class CacheManager {
 public:

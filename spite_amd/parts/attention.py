@@ -49,8 +49,8 @@ class Attention(Mixer):
                  qk_norm_first=False):
         if n_heads % n_kv_heads:
             raise ValueError(f"attention: {n_heads} heads over {n_kv_heads} kv heads")
-        if visibility not in ("full", "chunk", "window"):
-            raise ValueError(f"attention: visibility {visibility!r}")
+        if visibility not in hipops.VIS:
+            raise ValueError(f"attention: visibility {visibility!r} (known: {sorted(hipops.VIS)})")
         if visibility != "full" and span < 1:
             raise ValueError(f"attention: {visibility} of size {span}")
         self.env = env
