@@ -30,7 +30,7 @@ void attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_p
                         const bf16* __restrict__ v_pages, float* __restrict__ part, bf16* __restrict__ out,
                         const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                         const int* __restrict__ block_table, int max_blocks, int H, int G, int ps, int vis,
-                        int span, float scale_log2e, int n_splits) {
+                        int span, float scale_log2e, float cap_ratio, int n_splits) {
     constexpr int NC = HD / 32;      // 32-wide chunks of the head for the score product
     constexpr int ND = HD / 16;      // 16-row tiles of the output
     constexpr int ROW = HD + 2;      // partial record: output, max, sum
@@ -105,7 +105,10 @@ void attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_p
             for (int i = 0; i < 4; ++i) {
                 const int j = key0 + qd * 8 + tt * 4 + i;
                 ok[tt][i] = j >= lo && j <= p;
-                const float v = ok[tt][i] ? (page < 0 ? NAN : s[tt][i] * scale_log2e) : -INFINITY;
+                float raw = s[tt][i];
+                // a cap on the scores: cap * tanh(score * scale / cap), with cap_ratio = scale / cap
+                if (cap_ratio > 0.f) raw = tanhf(raw * cap_ratio) / cap_ratio;
+                const float v = ok[tt][i] ? (page < 0 ? NAN : raw * scale_log2e) : -INFINITY;
                 s[tt][i] = v;
                 mx = fmaxf(mx, v);
             }
@@ -223,7 +226,8 @@ extern "C" size_t spite_attn_decode_workspace(int T, int H, int hd, int n_splits
 extern "C" int spite_attn_decode(const void* q, const void* k_pages, const void* v_pages, void* out, void* workspace,
                                  const int* positions, const int* seq_of_token, const int* block_table,
                                  int max_blocks, int T, int H, int G, int hd, int page_size, int vis, int span,
-                                 float scale, int n_splits, hipStream_t st) {
+                                 float scale, float softcap, int n_splits, hipStream_t st) {
+    SP_REQUIRE(softcap >= 0.f && scale > 0.f, "attn_decode: scale %g, score cap %g", scale, softcap);
     SP_REQUIRE(T >= 0 && H > 0 && G > 0 && H % G == 0, "attn_decode: %d query heads over %d kv heads", H, G);
     SP_REQUIRE(H / G <= 16, "attn_decode: %d query heads per kv head, at most 16", H / G);
     SP_REQUIRE(hd == 64 || hd == 128, "attn_decode: head size %d (this kernel has 64 and 128)", hd);
@@ -232,18 +236,18 @@ extern "C" int spite_attn_decode(const void* q, const void* k_pages, const void*
     SP_REQUIRE(vis >= 0 && vis < SP_VIS_COUNT && (!sp_vis_has_span(vis) || span > 0), "attn_decode: chunk or window of %d", span);
     SP_REQUIRE(G <= 65535 && T <= 65535, "attn_decode: too many heads or tokens for one launch");
     if (T == 0) return 0;
-    const float sl = scale * 1.4426950408889634f;
+    const float sl = scale * 1.4426950408889634f, cr = softcap > 0.f ? scale / softcap : 0.f;
     dim3 grid(n_splits, G, T);
     const size_t sh = (size_t)4 * 16 * (hd + 2) * sizeof(float);
     if (hd == 128) {
         attn_decode_kernel<128><<<grid, 256, sh, st>>>((const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages,
-            (float*)workspace, (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, n_splits);
+            (float*)workspace, (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, cr, n_splits);
         SP_LAUNCH_CHECK("attn_decode");
         if (n_splits > 1)
             attn_decode_combine_kernel<128><<<dim3(T, H), 128, 0, st>>>((const float*)workspace, (bf16*)out, H, n_splits);
     } else {
         attn_decode_kernel<64><<<grid, 256, sh, st>>>((const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages,
-            (float*)workspace, (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, n_splits);
+            (float*)workspace, (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, cr, n_splits);
         SP_LAUNCH_CHECK("attn_decode");
         if (n_splits > 1)
             attn_decode_combine_kernel<64><<<dim3(T, H), 64, 0, st>>>((const float*)workspace, (bf16*)out, H, n_splits);
@@ -289,5 +293,5 @@ extern "C" int spite_attn_decode_static(const void* q, const void* k_pages, cons
     SP_REQUIRE(e == hipSuccess && ptr != nullptr, "attn_decode_static: no address for the scratch array: %s",
                hipGetErrorString(e));
     return spite_attn_decode(q, k_pages, v_pages, out, ptr, positions, seq_of_token, block_table, max_blocks, T, H, G,
-                             hd, page_size, vis, span, scale, n_splits, st);
+                             hd, page_size, vis, span, scale, 0.f, n_splits, st);
 }

@@ -15,7 +15,7 @@ __global__ __launch_bounds__(64)
 void attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
                          T* __restrict__ out, const int* __restrict__ positions,
                          const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
-                         int max_blocks, int H, int G, int hd, int ps, int vis, int span, float scale, int kv_tiled) {
+                         int max_blocks, int H, int G, int hd, int ps, int vis, int span, float scale, float softcap, int kv_tiled) {
     extern __shared__ float smem[];
     float* q_sh = smem;                 // [hd]
     float* p_sh = smem + hd;            // [64]
@@ -50,6 +50,7 @@ void attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
                 float acc = 0.f;
                 for (int c = 0; c < hd; ++c) acc = fmaf(q_sh[c], to_f32<T>(kr[sp_k_index(j % ps, c, hd, kv_tiled)]), acc);
                 s = acc * scale;
+                if (softcap > 0.f) s = softcap * tanhf(s / softcap);       // scores capped smoothly at +-softcap
             }
         }
         const float m_new = fmaxf(m, wave_max(s));
@@ -89,7 +90,8 @@ void attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
 extern "C" int spite_attn_generic(const void* q, const void* k_pages, const void* v_pages, void* out, int dtype,
                                   const int* positions, const int* seq_of_token, const int* block_table,
                                   int max_blocks, int T, int H, int G, int hd, int page_size, int vis, int span,
-                                  float scale, int kv_tiled, hipStream_t st) {
+                                  float scale, float softcap, int kv_tiled, hipStream_t st) {
+    SP_REQUIRE(softcap >= 0.f, "attention: score cap %g", softcap);
     SP_REQUIRE(T >= 0 && H > 0 && G > 0 && H % G == 0, "attention: %d query heads over %d kv heads", H, G);
     SP_REQUIRE(hd > 0 && hd <= 64 * ATT_MAX_D, "attention: head size %d, at most %d", hd, 64 * ATT_MAX_D);
     SP_REQUIRE(page_size > 0 && max_blocks > 0, "attention: bad page size %d or table width %d", page_size, max_blocks);
@@ -102,10 +104,10 @@ extern "C" int spite_attn_generic(const void* q, const void* k_pages, const void
     const size_t sh = (size_t)(hd + 64) * sizeof(float) + 64 * sizeof(long long) + 64 * sizeof(int) + 8;
     if (dtype == SP_F32)
         attn_generic_kernel<float><<<grid, 64, sh, st>>>((const float*)q, (const float*)k_pages, (const float*)v_pages,
-            (float*)out, positions, seq_of_token, block_table, max_blocks, H, G, hd, page_size, vis, span, scale, kv_tiled);
+            (float*)out, positions, seq_of_token, block_table, max_blocks, H, G, hd, page_size, vis, span, scale, softcap, kv_tiled);
     else if (dtype == SP_BF16)
         attn_generic_kernel<bf16><<<grid, 64, sh, st>>>((const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages,
-            (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, hd, page_size, vis, span, scale, kv_tiled);
+            (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, hd, page_size, vis, span, scale, softcap, kv_tiled);
     else return sp_fail("attention: unknown dtype %d", dtype);
     SP_LAUNCH_CHECK("attn_generic");
     return 0;

@@ -41,7 +41,7 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
                          const bf16* __restrict__ v_pages, bf16* __restrict__ out,
                          const int* __restrict__ positions, const int* __restrict__ cu_seqlens, int n_seqs,
                          const int* __restrict__ block_table, int max_blocks, int tile_q,
-                         int H, int G, int ps, int vis, int span, float scale_log2e) {
+                         int H, int G, int ps, int vis, int span, float scale_log2e, float cap_ratio) {
     constexpr int NC = HD / 32, ND = HD / 16;
     constexpr int KCH = KS * PF_KEYS * HD / 8 / 512; // 16-byte chunks of the step's K blocks per thread
     constexpr int VCH = KCH;                         // and of its V^T blocks
@@ -166,6 +166,17 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
                 for (int cc = 0; cc < NC; ++cc)
                     s[c][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[cc], qf[c][cc], s[c][tt], 0, 0, 0);
             }
+        }
+        if (cap_ratio > 0.f) {
+            // a cap on the scores: cap * tanh(score * scale / cap), with cap_ratio = scale / cap; the raw
+            // score is replaced by the one that the scale below turns into the capped score
+            const float inv = 1.0f / cap_ratio;
+#pragma unroll
+            for (int c = 0; c < 2; ++c)
+#pragma unroll
+                for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) s[c][tt][i] = tanhf(s[c][tt][i] * cap_ratio) * inv;
         }
         bf16x8 pf[2][2];
         float alpha[2];
@@ -302,7 +313,7 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
 template <int HD, int KS>
 static int launch_prefill(const void* q, const void* k_pages, const void* v_pages, void* out, const int* positions,
                           const int* cu_seqlens, int n_seqs, const int* block_table, int max_blocks, int tile_q,
-                          long n_tiles, int H, int G, int page_size, int vis, int span, float sl, hipStream_t st) {
+                          long n_tiles, int H, int G, int page_size, int vis, int span, float sl, float cr, hipStream_t st) {
     const size_t sh = (size_t)2 * 2 * KS * PF_KEYS * HD * sizeof(bf16);
     static bool allowed = false;          // one flag per instantiation: more LDS than the default limit
     if (!allowed) {
@@ -312,7 +323,7 @@ static int launch_prefill(const void* q, const void* k_pages, const void* v_page
     }
     attn_prefill_kernel<HD, KS><<<dim3((unsigned)n_tiles, G), 512, sh, st>>>((const bf16*)q, (const bf16*)k_pages,
         (const bf16*)v_pages, (bf16*)out, positions, cu_seqlens, n_seqs, block_table, max_blocks, tile_q, H, G, page_size,
-        vis, span, sl);
+        vis, span, sl, cr);
     SP_LAUNCH_CHECK("attn_prefill");
     return 0;
 }
@@ -323,7 +334,8 @@ static int launch_prefill(const void* q, const void* k_pages, const void* v_page
 extern "C" int spite_attn_prefill(const void* q, const void* k_pages, const void* v_pages, void* out,
                                   const int* positions, const int* cu_seqlens, const int* counts, int n_seqs,
                                   const int* block_table, int max_blocks, int H, int G, int hd, int page_size,
-                                  int vis, int span, float scale, int key_split, hipStream_t st) {
+                                  int vis, int span, float scale, float softcap, int key_split, hipStream_t st) {
+    SP_REQUIRE(softcap >= 0.f && scale > 0.f, "attn_prefill: scale %g, score cap %g", scale, softcap);
     SP_REQUIRE(n_seqs >= 0 && H > 0 && G > 0 && H % G == 0, "attn_prefill: %d query heads over %d kv heads", H, G);
     SP_REQUIRE(H / G <= PF_COLS / 2, "attn_prefill: %d query heads per kv head, at most %d", H / G, PF_COLS / 2);
     SP_REQUIRE(hd == 64 || hd == 128, "attn_prefill: head size %d (this kernel has 64 and 128)", hd);
@@ -344,10 +356,10 @@ extern "C" int spite_attn_prefill(const void* q, const void* k_pages, const void
     // few tiles: the longest tile's walk decides the time, so halve it
     if (key_split == 0) key_split = tiles[1] * G < 512 ? 2 : 1;
     SP_REQUIRE(tiles[key_split] <= 0x7fffffffL, "attn_prefill: too many tiles");
-    const float sl = scale * 1.4426950408889634f;
+    const float sl = scale * 1.4426950408889634f, cr = softcap > 0.f ? scale / softcap : 0.f;
     const int tile_q = PF_COLS / key_split / (H / G);
 #define SP_PF(HDV, KSV) launch_prefill<HDV, KSV>(q, k_pages, v_pages, out, positions, cu_seqlens, n_seqs, block_table, \
-        max_blocks, tile_q, tiles[KSV], H, G, page_size, vis, span, sl, st)
+        max_blocks, tile_q, tiles[KSV], H, G, page_size, vis, span, sl, cr, st)
     if (hd == 128) return key_split == 2 ? SP_PF(128, 2) : SP_PF(128, 1);
     return key_split == 2 ? SP_PF(64, 2) : SP_PF(64, 1);
 #undef SP_PF

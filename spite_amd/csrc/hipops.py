@@ -41,15 +41,15 @@ def lib():
             "spite_convert": [P, I, P, I, c_size_t, P],
             "spite_randn_fill": [P, I, c_size_t, ctypes.c_ulonglong, ctypes.c_ulonglong, F, F, P],
             "spite_gemm_generic": [P, I, P, L, I, P, I, I, I, I, I, P, I, P, P, P, I, P],
-            "spite_attn_generic": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, I, P],
+            "spite_attn_generic": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, F, I, P],
             "spite_sample_rows": [P, I, I, I, P, P, P, P],
             "spite_filter_rows": [P, I, I, I, P, P, P, P],
             "spite_gemm_skinny": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, I, I, I, P],
-            "spite_attn_decode": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, P],
+            "spite_attn_decode": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, F, I, P],
             "spite_gemm_mfma": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, P],
             "spite_gemm_tiled": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, P],
             "spite_gemm_tiled_split": [P, I, P, P, I, I, I, I, I, I, P, P],
-            "spite_attn_prefill": [P, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, F, I, P],
+            "spite_attn_prefill": [P, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, F, F, I, P],
             "spite_argmax_rows": [P, I, I, I, P, P, P, P],
             "spite_stream_read": [P, c_size_t, P, I, P],
         }
@@ -262,10 +262,11 @@ def gemm_generic(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_s
 
 
 def attn_generic(q, k_pages, v_pages, out, positions, seq_of_token, block_table, T, H, G, hd, page_size,
-                 vis, span, scale, kv_tiled=False):
+                 vis, span, scale, kv_tiled=False, softcap=0.0):
     """Attention over the paged cache, any mix of portions and single tokens.  q/out
     [T,H*hd]; block_table int32 [n_seqs, max_blocks].  ``kv_tiled``: the pages are in operand
-    order (``kv_operand_order``)."""
+    order (``kv_operand_order``).  ``softcap`` > 0 (here and in the MFMA kernels): the scaled scores
+    are capped smoothly, ``softcap * tanh(score / softcap)``, before the softmax."""
     if q.numel() < T * H * hd or out.numel() < T * H * hd:
         raise KernelError("attention: q or out too small")
     _check_pages(k_pages, v_pages, G, page_size, hd, "attention")
@@ -276,7 +277,7 @@ def attn_generic(q, k_pages, v_pages, out, positions, seq_of_token, block_table,
         _ptr(q, "q"), _ptr(k_pages, "k_pages", dt), _ptr(v_pages, "v_pages", dt), _ptr(out, "out", dt),
         dtype_code(dt), _ptr(positions, "positions", torch.int32), _ptr(seq_of_token, "seq_of_token", torch.int32),
         _ptr(block_table, "block_table", torch.int32), block_table.shape[1], T, H, G, hd, page_size,
-        VIS[vis], int(span or 0), float(scale), int(bool(kv_tiled)), _stream()), "attention")
+        VIS[vis], int(span or 0), float(scale), float(softcap), int(bool(kv_tiled)), _stream()), "attention")
 
 
 def sample_rows(logits, temperature, uniform, out, n_rows=None):
@@ -374,7 +375,7 @@ def attn_decode_workspace(T, H, hd, n_splits) -> int:
 
 
 def attn_decode(q, k_pages, v_pages, out, workspace, positions, seq_of_token, block_table, T, H, G, hd,
-                page_size, vis, span, scale, n_splits):
+                page_size, vis, span, scale, n_splits, softcap=0.0):
     """Split-KV decode attention on MFMA (bf16; head sizes 64 and 128; pages of a multiple of 32
     keys, in operand order): every row of q is one query against its request's cache."""
     if q.dtype != torch.bfloat16:
@@ -391,8 +392,8 @@ def attn_decode(q, k_pages, v_pages, out, workspace, positions, seq_of_token, bl
         _ptr(q, "q", dt), _ptr(k_pages, "k_pages", dt), _ptr(v_pages, "v_pages", dt), _ptr(out, "out", dt),
         _ptr(workspace, "workspace"), _ptr(positions, "positions", torch.int32),
         _ptr(seq_of_token, "seq_of_token", torch.int32), _ptr(block_table, "block_table", torch.int32),
-        block_table.shape[1], T, H, G, hd, page_size, VIS[vis], int(span or 0), float(scale), int(n_splits),
-        _stream()), "attn_decode")
+        block_table.shape[1], T, H, G, hd, page_size, VIS[vis], int(span or 0), float(scale), float(softcap),
+        int(n_splits), _stream()), "attn_decode")
 
 
 def gemm_mfma(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None, glu=False,
@@ -460,7 +461,7 @@ def gemm_tiled(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_sca
 
 
 def attn_prefill(q, k_pages, v_pages, out, positions, cu_seqlens, counts, block_table,
-                 H, G, hd, page_size, vis, span, scale, key_split=0):
+                 H, G, hd, page_size, vis, span, scale, key_split=0, softcap=0.0):
     """Prefill attention on MFMA (bf16; head sizes 64 and 128; pages of a multiple of 32 keys, in
     operand order).
     ``counts``: the number of query tokens of every request of the step, on the host, in the
@@ -482,7 +483,8 @@ def attn_prefill(q, k_pages, v_pages, out, positions, cu_seqlens, counts, block_
         _ptr(q, "q", dt), _ptr(k_pages, "k_pages", dt), _ptr(v_pages, "v_pages", dt), _ptr(out, "out", dt),
         _ptr(positions, "positions", torch.int32), _ptr(cu_seqlens, "cu_seqlens", torch.int32),
         counts.ctypes.data, n_seqs, _ptr(block_table, "block_table", torch.int32), block_table.shape[1],
-        H, G, hd, page_size, VIS[vis], int(span or 0), float(scale), int(key_split), _stream()), "attn_prefill")
+        H, G, hd, page_size, VIS[vis], int(span or 0), float(scale), float(softcap), int(key_split), _stream()),
+        "attn_prefill")
 
 
 def argmax_rows(logits, out, scratch_v, scratch_i, n_rows=None):

@@ -46,7 +46,7 @@ class Attention(Mixer):
 
     def __init__(self, env, hidden_size, n_heads, n_kv_heads, head_dim, position, visibility="full", span=0,
                  qk_norm=False, qk_norm_eps=1e-5, temperature=None, softmax_scale=None, qk_norm_weighted=False,
-                 qk_norm_first=False):
+                 qk_norm_first=False, score_cap=None):
         if n_heads % n_kv_heads:
             raise ValueError(f"attention: {n_heads} heads over {n_kv_heads} kv heads")
         if visibility not in hipops.VIS:
@@ -56,6 +56,10 @@ class Attention(Mixer):
         self.env = env
         self.d, self.H, self.G, self.hd = int(hidden_size), int(n_heads), int(n_kv_heads), int(head_dim)
         self.visibility, self.span = visibility, int(span or 0)
+        # scaled scores capped smoothly before the softmax, cap * tanh(score / cap); None: no cap
+        self.score_cap = float(score_cap or 0.0)
+        if self.score_cap < 0:
+            raise ValueError(f"attention: score cap {score_cap}")
         self.qk_norm, self.qk_norm_eps = bool(qk_norm), float(qk_norm_eps)
         # the head norm's weights ([hd] each for queries and keys) and its place: after the rotation
         # (Llama 4, weightless) or before it
@@ -106,7 +110,7 @@ class Attention(Mixer):
         scratch = ctx.ws.take((hipops.attn_decode_workspace(T, H, hd, n_splits) // 4,), torch.float32)
         hipops.attn_decode(q, cache.k_pages, cache.v_pages, o, scratch, ctx.positions, ctx.seq_of_token,
                            cache.block_table, T, H, G, hd, cache.page_size, self.visibility, self.span,
-                           self.scale, n_splits)
+                           self.scale, n_splits, softcap=self.score_cap)
 
     def forward(self, x, ctx, cache):
         T = x.shape[0]
@@ -138,14 +142,15 @@ class Attention(Mixer):
                 self._decode(q, o, ctx, cache, lead)
                 hipops.attn_prefill(q[lead:], cache.k_pages, cache.v_pages, o[lead:], ctx.positions[lead:], cu_tail,
                                     ctx.host.counts[lead:], cache.block_table[lead:], H, G, hd, cache.page_size,
-                                    self.visibility, self.span, self.scale)
+                                    self.visibility, self.span, self.scale, softcap=self.score_cap)
             else:
                 hipops.attn_prefill(q, cache.k_pages, cache.v_pages, o, ctx.positions, ctx.cu_seqlens, ctx.host.counts,
-                                    cache.block_table, H, G, hd, cache.page_size, self.visibility, self.span, self.scale)
+                                    cache.block_table, H, G, hd, cache.page_size, self.visibility, self.span, self.scale,
+                                    softcap=self.score_cap)
         else:
             hipops.attn_generic(q, cache.k_pages, cache.v_pages, o, ctx.positions, ctx.seq_of_token,
                                 cache.block_table, T, H, G, hd, cache.page_size, self.visibility, self.span,
-                                self.scale, kv_tiled=cache.tiled)
+                                self.scale, kv_tiled=cache.tiled, softcap=self.score_cap)
         out = ws.take((T, self.d), torch.float32)
         linear(o, self.wo, out, ws=ws)
         return out

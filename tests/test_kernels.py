@@ -401,8 +401,9 @@ class PagedKV:
             self.bt[s, b] = -1
 
 
-def attention_reference(kv, queries, qs, H, vis, span):
-    """queries: list of (request, position); qs [T,H,hd]."""
+def attention_reference(kv, queries, qs, H, vis, span, softcap=0.0):
+    """queries: list of (request, position); qs [T,H,hd].  ``softcap``: the scaled scores are
+    capped, softcap * tanh(score / softcap), before the softmax."""
     out = torch.zeros(len(queries), H, kv.hd, dtype=torch.float64)
     for t, (s, p) in enumerate(queries):
         pos = torch.arange(p + 1)
@@ -410,15 +411,25 @@ def attention_reference(kv, queries, qs, H, vis, span):
             mask = plain.visible_mask(pos, vis, span)[p:p + 1]
         else:                        # the whole square would not fit: the query's own row of it
             mask = (pos >= plain_first(vis, span, p)).view(1, -1)
-        out[t] = plain.attention(qs[t:t + 1].double(), kv.k[s][:p + 1].double(), kv.v[s][:p + 1].double(), mask)[0]
+        if not softcap:
+            out[t] = plain.attention(qs[t:t + 1].double(), kv.k[s][:p + 1].double(), kv.v[s][:p + 1].double(), mask)[0]
+            continue
+        k, v = kv.k[s][:p + 1].double(), kv.v[s][:p + 1].double()          # [keys, G, hd]
+        for h in range(H):
+            g = h // (H // k.shape[1])
+            score = (k[:, g] @ qs[t, h].double()) / math.sqrt(kv.hd)
+            score = softcap * torch.tanh(score / softcap)
+            score = score.masked_fill(~mask[0], float("-inf"))
+            out[t, h] = torch.softmax(score, 0) @ v[:, g]
     return out
 
 
-def run_attention(kind, dtype, H, G, hd, ps, lens, queries, vis, span, n_splits=3, seed=0, planted=None):
+def run_attention(kind, dtype, H, G, hd, ps, lens, queries, vis, span, n_splits=3, seed=0, planted=None, softcap=0.0,
+                  q_gain=1.0):
     kv = PagedKV(lens, G, hd, ps, dtype, seed)
     T = len(queries)
     g = torch.Generator().manual_seed(seed + 1)
-    qs = torch.randn(T, H, hd, generator=g).to(dtype)
+    qs = (torch.randn(T, H, hd, generator=g) * q_gain).to(dtype)
     if planted is not None:                      # one far key that the query must find
         t, s, j = planted
         kv.k[s][j] = (qs[t, ::H // G] * 3.0).to(dtype)
@@ -428,7 +439,7 @@ def run_attention(kind, dtype, H, G, hd, ps, lens, queries, vis, span, n_splits=
                                for s in range(len(lens))]):
         low = min([plain_first(vis, span, p) for ss, p in queries if ss == s], default=0)
         kv.drop_below(s, low)
-    ref = attention_reference(kv, queries, qs, H, vis, span)
+    ref = attention_reference(kv, queries, qs, H, vis, span, softcap)
     positions = torch.tensor([p for _, p in queries], dtype=torch.int32, device=DEV)
     seq = torch.tensor([s for s, _ in queries], dtype=torch.int32, device=DEV)
     out = torch.zeros(T, H * hd, dtype=dtype, device=DEV)
@@ -437,11 +448,12 @@ def run_attention(kind, dtype, H, G, hd, ps, lens, queries, vis, span, n_splits=
     if kind != "generic":                        # the MFMA kernels read pages in operand order
         kp, vp = ops().kv_operand_order(kp, vp)
     if kind == "generic":
-        ops().attn_generic(q_dev, kp, vp, out, positions, seq, bt, T, H, G, hd, ps, vis, span, scale)
+        ops().attn_generic(q_dev, kp, vp, out, positions, seq, bt, T, H, G, hd, ps, vis, span, scale, softcap=softcap)
         if ops().kv_tiled_ok(dtype, hd, ps):     # and the plain kernel reads them too, with the same bits
             again = torch.zeros_like(out)
             kpt, vpt = ops().kv_operand_order(kp, vp)
-            ops().attn_generic(q_dev, kpt, vpt, again, positions, seq, bt, T, H, G, hd, ps, vis, span, scale, kv_tiled=True)
+            ops().attn_generic(q_dev, kpt, vpt, again, positions, seq, bt, T, H, G, hd, ps, vis, span, scale, kv_tiled=True,
+                               softcap=softcap)
             assert torch.equal(out, again)
     elif kind == "prefill":                      # runs of queries of one request are the portions
         runs = []
@@ -452,11 +464,12 @@ def run_attention(kind, dtype, H, G, hd, ps, lens, queries, vis, span, n_splits=
                 runs.append([s, 1])
         cu = torch.tensor([0] + list(np.cumsum([c for _, c in runs])), dtype=torch.int32, device=DEV)
         ops().attn_prefill(q_dev, kp, vp, out, positions, cu, [c for _, c in runs],
-                           bt[[s for s, _ in runs]].contiguous(), H, G, hd, ps, vis, span, scale)
+                           bt[[s for s, _ in runs]].contiguous(), H, G, hd, ps, vis, span, scale, softcap=softcap)
     else:
         wsz = ops().attn_decode_workspace(T, H, hd, n_splits)
         scratch = torch.empty(wsz // 4, dtype=torch.float32, device=DEV)
-        ops().attn_decode(q_dev, kp, vp, out, scratch, positions, seq, bt, T, H, G, hd, ps, vis, span, scale, n_splits)
+        ops().attn_decode(q_dev, kp, vp, out, scratch, positions, seq, bt, T, H, G, hd, ps, vis, span, scale, n_splits,
+                          softcap=softcap)
     got = out.double().cpu().view(T, H, hd)
     err = (got - ref).abs().max()
     assert torch.isfinite(got).all()
@@ -544,6 +557,26 @@ def test_attn_prefill(case, key_split):
     got = out.double().cpu().view(T, H, hd)
     assert torch.isfinite(got).all()
     assert (got - ref).abs().max() < 1.5e-2 * max(1.0, float(ref.abs().max()))
+
+
+@pytest.mark.parametrize("kind,dtype", [("generic", torch.float32), ("generic", torch.bfloat16), ("decode", torch.bfloat16),
+                                        ("prefill", torch.bfloat16)])
+def test_attention_with_capped_scores(kind, dtype):
+    """Scores capped smoothly before the softmax (an option of every attention kernel): queries
+    three times as long as usual, so that scores reach beyond the cap of 4 and the cap matters."""
+    H, G, hd, ps = (8, 2, 128, 64) if kind != "generic" else (6, 3, 24, 8)
+    queries = [(0, p) for p in range(250, 300)] if kind == "prefill" else [(0, 299), (1, 128), (0, 40)]
+    if kind == "prefill":
+        queries += [(1, p) for p in range(0, 129)]
+    else:
+        queries = sorted(queries)
+    got, ref = run_attention(kind, dtype, H, G, hd, ps, [300, 129], queries, "chunk", 128, softcap=4.0, q_gain=3.0)
+    # without the cap the result is another one
+    kv = PagedKV([300, 129], G, hd, ps, dtype, 0)
+    g = torch.Generator().manual_seed(1)
+    qs = (torch.randn(len(queries), H, hd, generator=g) * 3.0).to(dtype)
+    other = attention_reference(kv, queries, qs, H, "chunk", 128)
+    assert (other - ref).abs().max() > 0.1
 
 
 def test_prefill_attention_finds_one_far_key_among_thousands():

@@ -374,10 +374,10 @@ def test_other_ends_of_a_model_an_embedding_with_a_scale_and_a_head_with_a_cap_a
     assert abs(ref).max() > 1.5            # the cap is felt
 
 
-def test_attention_with_a_weighted_head_norm_before_a_rotation_of_part_of_the_head():
+def test_attention_with_a_weighted_head_norm_before_a_rotation_of_part_of_the_head_and_capped_scores():
     """What other architectures' attention needs beside Llama 4's: the head norm with weights, placed
-    before the rotation, and a rotation of the head's first elements only - options of the built-in
-    mixer and position encoding, chosen by the spec."""
+    before the rotation, a rotation of the head's first elements only, and scores capped smoothly
+    before the softmax - options of the built-in mixer and position encoding, chosen by the spec."""
     from spite_amd import Engine
     from spite_amd.parts import PartSpec, BlockSpec, LayerCall, ModelSpec
     import plain_llama4 as plain
@@ -386,7 +386,7 @@ def test_attention_with_a_weighted_head_norm_before_a_rotation_of_part_of_the_he
     names = {k: f"b1.attn.{k}" for k in ("q_proj", "k_proj", "v_proj", "o_proj")}
     names.update(q_norm="b1.attn.q_norm", k_norm="b1.attn.k_norm")
     attn = PartSpec("attention", dict(hidden_size=D, n_heads=HEADS, n_kv_heads=KV, head_dim=HD, qk_norm=True, qk_norm_eps=1e-6,
-                                      qk_norm_weighted=True, qk_norm_first=True,
+                                      qk_norm_weighted=True, qk_norm_first=True, score_cap=1.5,
                                       position=PartSpec("rotary", {"head_dim": HD, "theta": 100.0, "rotary_dim": rot})), names)
     dense = PartSpec("dense_glu", {"hidden_size": D, "intermediate_size": 40},
                      {k: f"b1.ffn.{k}" for k in ("gate_proj", "up_proj", "down_proj")})
@@ -409,7 +409,13 @@ def test_attention_with_a_weighted_head_norm_before_a_rotation_of_part_of_the_he
     q = rotate(plain.rms_norm((n @ W["b1.attn.q_proj"].T).view(T, HEADS, HD), W["b1.attn.q_norm"], 1e-6))
     k = rotate(plain.rms_norm((n @ W["b1.attn.k_proj"].T).view(T, KV, HD), W["b1.attn.k_norm"], 1e-6))
     v = (n @ W["b1.attn.v_proj"].T).view(T, KV, HD)
-    h = h + plain.attention(q, k, v, plain.visible_mask(pos, "full", 0)).reshape(T, HEADS * HD) @ W["b1.attn.o_proj"].T
+    mask, att = plain.visible_mask(pos, "full", 0), torch.zeros(T, HEADS, HD, dtype=torch.float64)
+    for hh in range(HEADS):
+        score = q[:, hh] @ k[:, hh // (HEADS // KV)].T / HD ** 0.5
+        score = (1.5 * torch.tanh(score / 1.5)).masked_fill(~mask, float("-inf"))
+        att[:, hh] = torch.softmax(score, -1) @ v[:, hh // (HEADS // KV)]
+    assert (att - plain.attention(q, k, v, mask)).abs().max() > 0.02          # the cap matters here
+    h = h + att.reshape(T, HEADS * HD) @ W["b1.attn.o_proj"].T
     h = h + plain.swiglu_mlp(plain.rms_norm(h, W["b1.n2"], 1e-5), W["b1.ffn.gate_proj"], W["b1.ffn.up_proj"], W["b1.ffn.down_proj"])
     ref = (plain.rms_norm(h, W["final"], 1e-5) @ W["head"].T).float().numpy()
     reqs = {"x": toks}
