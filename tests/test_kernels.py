@@ -155,6 +155,20 @@ def test_rope_kvwrite_with_part_of_the_head_rotating_and_a_weighted_norm_before_
     for t in range(T):
         page, off = int(slots[t]) // ps, int(slots[t]) % ps
         assert (kp[page, :, off].double().cpu() - want_k[t]).abs().max() < tol
+    if ops().kv_tiled_ok(dtype, hd, 32):       # the same rows into pages of 32, row-major and in operand order
+        kp32, vp32 = torch.zeros(n_pages, G, 32, hd, dtype=dtype, device=DEV), torch.zeros(n_pages, G, hd, 32, dtype=dtype, device=DEV)
+        kpt, vpt, q2 = torch.zeros_like(kp32), torch.zeros_like(vp32), torch.empty_like(q)
+        slots32 = (slots // ps) * 32 + ((slots % ps) * 9 + (slots // ps)) % 32
+        for tiled, (a, b) in ((False, (kp32, vp32)), (True, (kpt, vpt))):
+            ops().rope_kvwrite(qkv, q2, a, b, pos, slots32, inv, H, G, hd, 32, use_rope=True, adjacent=adjacent, use_norm=True,
+                               norm_eps=1e-5, use_temp=False, floor_scale=1, attn_scale=0.0, rotary_dim=rot,
+                               norm_weight_q=wq, norm_weight_k=wk, norm_first=first, kv_tiled=tiled)
+            assert torch.equal(q2, q)
+        want_kt, want_vt = ops().kv_operand_order(kp32, vp32)
+        assert float(kp32.abs().sum()) > 0 and torch.equal(kpt, want_kt) and torch.equal(vpt, want_vt)
+        for t in range(T):
+            page, off = int(slots32[t]) // 32, int(slots32[t]) % 32
+            assert (kp32[page, :, off].double().cpu() - want_k[t]).abs().max() < tol
     # a wrong order of norm and rotation shows where the weights are not all alike
     if weighted:
         other_q = norm(rotate(qq), wq) if first else rotate(norm(qq, wq))
