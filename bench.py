@@ -106,8 +106,8 @@ class Sizes:
 
 def measured_peaks(dtype):
     """What this GPU gives to the simplest kernels of the same kind: a streaming read of 4 GiB
-    (non-temporal loads, a contiguous piece per workgroup) and this library's dense product at
-    8192^3, the best of five runs each."""
+    (non-temporal loads, a contiguous piece per workgroup), this library's dense product at
+    8192^3, and a loop of MFMAs alone on random and on zero operands; the best of a few runs each."""
     import torch
     from spite_amd.csrc import hipops
     dev = torch.device("cuda:0")
@@ -136,6 +136,18 @@ def measured_peaks(dtype):
             torch.cuda.synchronize()
             rate = max(rate, 2.0 * n ** 3 / (time.perf_counter() - t))
         res["dense_product_TFLOPs"] = round(rate / 1e12, 1)
+        # the matrix units alone, operands in registers: on pseudo-random values and on zeros (the
+        # difference is the chip's power limit, which real values meet and zeros do not)
+        out = torch.zeros(1024, dtype=torch.float32, device=dev)
+        for label, gain in (("mfma_loop_random_TFLOPs", 1.0), ("mfma_loop_zeros_TFLOPs", 0.0)):
+            rate = 0.0
+            for _ in range(3):
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+                flops = hipops.mfma_loop(out, 4000, gain)
+                torch.cuda.synchronize()
+                rate = max(rate, flops / (time.perf_counter() - t))
+            res[label] = round(rate / 1e12, 1)
     torch.cuda.empty_cache()
     return res
 
@@ -436,6 +448,8 @@ def main() -> int:
                    "runs_ms": [round(x * 1e3, 3) for x in pre_runs]}
         if peaks and "dense_product_TFLOPs" in peaks:
             prefill["frac_of_measured_product"] = round(pf / pre / (peaks["dense_product_TFLOPs"] * 1e12), 4)
+        if peaks and "mfma_loop_random_TFLOPs" in peaks:
+            prefill["frac_of_mfma_on_random_values"] = round(pf / pre / (peaks["mfma_loop_random_TFLOPs"] * 1e12), 4)
         if args.prefill_context:
             prefill["after"] = args.prefill_context
         log(f"prefill {args.prefill_tokens} tokens" + (f" after {args.prefill_context}" if args.prefill_context else "")

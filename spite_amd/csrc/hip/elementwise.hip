@@ -816,3 +816,52 @@ extern "C" int spite_stream_read(const void* p, size_t nbytes, float* out, int n
     SP_LAUNCH_CHECK("stream_read");
     return 0;
 }
+
+// ------------------------------------------------------------------ the matrix units alone, for measurement
+// 32 independent MFMA 16x16x32 a step on operands that stay in registers: what the chip gives to the
+// products when nothing else moves.  `gain` scales the operands' pseudo-random values; with 0 nothing
+// toggles, and the rate shows how much of the time under real values is the chip's power limit.
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void mfma_loop_kernel(float* __restrict__ out, int steps, float gain) {
+    const unsigned id = blockIdx.x * 512 + threadIdx.x;
+    auto operand = [&](unsigned seed) {
+        bf16x8 v;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            unsigned x = (id * 16 + seed) * 8 + e;
+            x ^= x >> 16; x *= 0x7feb352dU; x ^= x >> 15; x *= 0x846ca68bU; x ^= x >> 16;
+            v[e] = (bf16)(((int)(x & 0xffff) - 32768) / 32768.0f * gain);
+        }
+        return v;
+    };
+    bf16x8 a[4], b[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) a[i] = operand(i);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) b[i] = operand(4 + i);
+    f32x4 acc[4][8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < steps; ++t) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s += acc[i][j][0] + acc[i][j][3];
+    if (threadIdx.x == 0) out[blockIdx.x] = s;
+}
+
+// Runs `n_blocks` workgroups of eight waves, each wave `steps` times 32 MFMAs of 16,384 flops.
+extern "C" int spite_mfma_loop(float* out, int n_blocks, int steps, float gain, hipStream_t st) {
+    SP_REQUIRE(n_blocks > 0 && steps > 0 && out, "mfma_loop: %d workgroups, %d steps", n_blocks, steps);
+    mfma_loop_kernel<<<n_blocks, 512, 0, st>>>(out, steps, gain);
+    SP_LAUNCH_CHECK("mfma_loop");
+    return 0;
+}

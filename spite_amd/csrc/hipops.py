@@ -52,6 +52,7 @@ def lib():
             "spite_attn_prefill": [P, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, F, F, I, P],
             "spite_argmax_rows": [P, I, I, I, P, P, P, P],
             "spite_stream_read": [P, c_size_t, P, I, P],
+            "spite_mfma_loop": [P, I, I, F, P],
         }
         for name, args in sigs.items():
             fn = getattr(l, name)
@@ -507,3 +508,11 @@ def stream_read(t, out):
         raise KernelError("stream_read: out holds eight floats per workgroup")
     _check(lib().spite_stream_read(_ptr(t, "t"), nbytes - nbytes % 16, _ptr(out, "out", torch.float32), out.numel() // 8,
                                    _stream()), "stream_read")
+
+
+def mfma_loop(out, steps, gain):
+    """Runs ``out.numel()`` workgroups of eight waves, every wave ``steps`` times 32 MFMA 16x16x32 on
+    operands in registers (pseudo-random values scaled by ``gain``; 0: all zero): the matrix units'
+    rate with nothing else moving.  Returns the flops done."""
+    _check(lib().spite_mfma_loop(_ptr(out, "out", torch.float32), out.numel(), int(steps), float(gain), _stream()), "mfma_loop")
+    return out.numel() * 8 * int(steps) * 32 * 16384

@@ -871,3 +871,14 @@ def test_randn_fill_equals_its_host_port_bit_for_bit():
         h = torch.empty(n, dtype=torch.bfloat16, device=DEV)
         ops().randn_fill(h, seed, key, mean, std)
         assert torch.equal(h.cpu(), torch.from_numpy(host).to(torch.bfloat16))
+
+
+def test_mfma_loop_runs_and_counts_its_flops():
+    """The benchmark's loop of MFMAs alone: it finishes, writes a sum per workgroup, and on zero
+    operands every sum is zero."""
+    out = torch.full((8,), -1.0, device=DEV)
+    flops = ops().mfma_loop(out, 10, 0.0)
+    torch.cuda.synchronize()
+    assert flops == 8 * 8 * 10 * 32 * 16384 and float(out.abs().sum()) == 0.0
+    ops().mfma_loop(out, 10, 1.0)
+    assert torch.isfinite(out).all() and float(out.abs().sum()) > 0.0
