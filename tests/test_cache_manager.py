@@ -220,3 +220,24 @@ def test_a_chunked_group_gets_no_more_pages_than_its_requests_can_hold():
     # small pools are left as they are
     small = PagedCache(needs[:2], 16, 8, 4, torch.float32, torch.device("cpu"), allocate=False, portion=2048)
     assert [small.total_pages(g) for g in range(2)] == [8, 8]
+
+
+def test_the_visibility_rules_have_one_definition():
+    """The names and codes of the rules that say which keys a query reads come from one header;
+    the cache manager (native) frees exactly what that header's rule no longer reads."""
+    from spite_amd.csrc import build, hipops, hostlib
+    from spite_amd.cache import paged
+    codes = build.visibility_codes()
+    assert codes == {"full": 0, "chunk": 1, "window": 2} and hipops.VIS == codes and paged._KINDS == codes
+    lib = hostlib.lib()
+    for kind, span, n, first in (("full", 0, 37, 0), ("chunk", 8, 37, 32), ("window", 8, 37, 30), ("window", 8, 5, 0)):
+        h = lib.spc_create(4, 1, 1, hostlib.int_array([codes[kind]]), hostlib.int_array([span]), hostlib.int_array([32]))
+        s = lib.spc_admit(h)
+        assert lib.spc_reserve(h, s, n) == 0 and lib.spc_commit(h, s, n) == 0
+        n_tab = lib.spc_table_len(h, s, 0)
+        tab = hostlib.int_array([0] * n_tab)
+        lib.spc_table(h, s, 0, tab, n_tab)
+        held = [i for i in range(n_tab) if tab[i] >= 0]
+        # the next query (position n) reads from `first`: pages wholly below it are gone
+        assert held == list(range(first // 4, -(-n // 4))), (kind, span, held)
+        lib.spc_destroy(h)
