@@ -343,20 +343,21 @@ class Engine:
                 segments.append((lo, hi, None, {"before": before, "marks": marks, "addresses": self._addresses(state)}))
                 continue
             graph = torch.cuda.CUDAGraph()
+            before, marks = dict(state), tuple(ws.mark() for ws in (*self._arenas, self._step_ws))
             try:
                 with torch.cuda.graph(graph):
                     self._run_eager(lo, hi, state, meta)
             except Exception:
-                # nothing of this segment has run yet (a capture computes nothing): the rest of the
-                # step runs eagerly, and so does every later step, loudly
+                # nothing of this segment has run yet (a capture computes nothing): what the units
+                # took and handed on while they were recorded is put back, the rest of the step
+                # runs eagerly, and so does every later step, loudly
                 self._graphs.pop(key, None)
                 self.use_graphs = False
                 import warnings
                 warnings.warn("capturing the decode step in a HIP graph failed; steps run eagerly from now on")
-                if lo == 0:
-                    self._step_ws.reset()
-                    state = {}
-                return self._run_eager(lo, self.model.n_units(), state, meta)["logits"]
+                for ws, mark in zip((*self._arenas, self._step_ws), marks):
+                    ws.rewind(mark)
+                return self._run_eager(lo, self.model.n_units(), before, meta)["logits"]
             if self._drop_stale_graphs():  # cannot happen (a workspace refuses to grow under capture)
                 self._graphs.pop(key, None)
                 return self._run_eager(lo, self.model.n_units(), state, meta)["logits"]

@@ -85,3 +85,83 @@ def test_a_graph_is_not_replayed_after_a_later_step_has_moved_the_workspaces(tmp
         eng.cache.check()
     for a, b in zip(*outs):
         assert a.shape == b.shape and np.array_equal(a, b)
+
+
+def test_a_capture_that_fails_midway_falls_back_to_eager_steps_with_the_right_logits():
+    """A part that says it can be captured and cannot (it reads a value back on the host): the
+    capture fails in the middle of the model.  What the recorded units took and handed on is put
+    back, the step is finished eagerly with a warning, later steps run eagerly, and every logit
+    equals the eager engine's."""
+    import torch
+    from spite_amd import Engine, StepEntry
+    from spite_amd.parts import Mixer, ParamSpec, CacheNeed, register, PartSpec, BlockSpec, LayerCall, ModelSpec
+
+    @register("mixer", "toy_claims_to_be_safe")
+    class ClaimsToBeSafe(Mixer):
+        graph_safe = True
+
+        def __init__(self, env, width):
+            self.width, self.w = width, None
+
+        def params(self):
+            return {"proj": ParamSpec((self.width, self.width))}
+
+        def load(self, tensors):
+            self.w = tensors["proj"]
+
+        def cache_need(self):
+            return CacheNeed()
+
+        def forward(self, x, ctx, cache):
+            gain = 1.0 + 0.0 * float(x[0, 0])              # a read-back: refused while a graph is recorded
+            out = ctx.ws.take((ctx.T, self.width), torch.float32)
+            torch.matmul(x.float() * gain, self.w.float().T, out=out)
+            return out
+
+    @register("mixer", "toy_reads_the_step_on_the_host")
+    class ReadsTheHost(ClaimsToBeSafe):
+        graph_safe = False
+
+        def forward(self, x, ctx, cache):
+            assert int(ctx.host.counts.sum()) == ctx.T           # the step's metadata, on the host
+            out = ctx.ws.take((ctx.T, self.width), torch.float32)
+            torch.matmul(x.float(), self.w.float().T, out=out)
+            return out
+
+    D, V = 32, 50
+    g = torch.Generator().manual_seed(4)
+    r = lambda *s: torch.randn(*s, generator=g) * 0.3
+    norm = lambda name: PartSpec("rms", {"width": D, "eps": 1e-5}, {"weight": name})
+    ffn = lambda p: PartSpec("dense_glu", {"hidden_size": D, "intermediate_size": 48}, {k: f"{p}.{k}" for k in ("gate_proj", "up_proj", "down_proj")})
+    attn = lambda p: PartSpec("attention", dict(hidden_size=D, n_heads=2, n_kv_heads=1, head_dim=16,
+                                                position=PartSpec("rotary", {"head_dim": 16, "theta": 100.0})),
+                              {k: f"{p}.{k}" for k in ("q_proj", "k_proj", "v_proj", "o_proj")})
+    # an honest eager unit first, so that the failing capture starts in the middle of the step
+    blocks = [BlockSpec("prenorm", norm("b0.n1"), PartSpec("toy_reads_the_step_on_the_host", {"width": D}, {"proj": "b0.mix"}), norm("b0.n2"), ffn("b0.ffn")),
+              BlockSpec("prenorm", norm("b1.n1"), PartSpec("toy_claims_to_be_safe", {"width": D}, {"proj": "b1.mix"}), norm("b1.n2"), ffn("b1.ffn")),
+              BlockSpec("prenorm", norm("b2.n1"), attn("b2.attn"), norm("b2.n2"), ffn("b2.ffn"))]
+    sp = ModelSpec("ToyFails", V, D, blocks, [LayerCall(0, 0), LayerCall(1, 1), LayerCall(2, 2)], norm("final"), "embed", "head")
+    t = {"embed": r(V, D), "head": r(V, D), "final": 1 + r(D) * 0.1, "b1.mix": r(D, D), "b0.mix": r(D, D)}
+    for b in range(3):
+        t[f"b{b}.n1"], t[f"b{b}.n2"] = 1 + r(D) * 0.1, 1 + r(D) * 0.1
+        t[f"b{b}.ffn.gate_proj"], t[f"b{b}.ffn.up_proj"], t[f"b{b}.ffn.down_proj"] = r(48, D), r(48, D), r(D, 48)
+    for b in (2,):
+        t[f"b{b}.attn.q_proj"], t[f"b{b}.attn.o_proj"] = r(32, D), r(D, 32)
+        t[f"b{b}.attn.k_proj"], t[f"b{b}.attn.v_proj"] = r(16, D), r(16, D)
+    outs = []
+    for graphs in (True, False):
+        eng = Engine(spec=sp, tensors=t, dtype="float32", page_size=4, cache_tokens=64, max_requests=2, graphs=graphs)
+        assert [safe for _, _, safe in eng.model.graph_segments()] == [True, False, True]
+        s = eng.admit()
+        eng.step([StepEntry(s, [1, 2, 3], [])])
+        rows = [eng.step([StepEntry(s, [4], [0])]).cpu().clone()]               # first decode step: eager
+        if graphs:
+            with pytest.warns(UserWarning, match="capturing"):
+                rows.append(eng.step([StepEntry(s, [5], [0])]).cpu().clone())    # second: the capture fails midway
+            assert not eng.use_graphs and eng.graph_replays == 0
+        else:
+            rows.append(eng.step([StepEntry(s, [5], [0])]).cpu().clone())
+        rows += [eng.step([StepEntry(s, [6 + i], [0])]).cpu().clone() for i in range(4)]
+        outs.append(rows)
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
