@@ -89,7 +89,7 @@ class PagedCache:
                 for g, n in zip(self.groups, pages):
                     g.n_pages = n
                 self._h = create()
-        self._fresh_buf = (ctypes.c_int * (4 * self.max_requests + 4))()
+        self._fresh_buf = (ctypes.c_int * self.max_requests)()
         self.states: Dict[int, torch.Tensor] = {}
         if allocate:
             for g in self.groups:
@@ -128,11 +128,9 @@ class PagedCache:
         whomever (this object's ``admit`` or the native scheduler, which admits on its own): the
         step function calls it before it runs, so a new request never meets the state that the
         slot's last request left.  Returns those slots."""
+        # each slot is reported once however often it changed hands: never more than there are slots
         n = self._lib.spc_take_fresh(self._h, self._fresh_buf, len(self._fresh_buf))
-        if n > len(self._fresh_buf):           # more admissions than slots since the last step: clear them all
-            slots = list(range(self.max_requests))
-        else:
-            slots = sorted(set(self._fresh_buf[:n]))
+        slots = list(self._fresh_buf[:n])
         if slots:
             for st in self.states.values():
                 st[slots] = 0
@@ -154,6 +152,18 @@ class PagedCache:
                              f"{[self.free_pages(g) for g in range(self.n_groups())]}")
         if rc != 0:
             raise CacheError(f"reserve: slot {slot} is not live")
+
+    def reserve_all(self, pairs):
+        """``reserve`` for every ``(slot, n)`` of a step: all of them get their pages, or nothing
+        changes and ``OutOfPages`` says so."""
+        slots = (ctypes.c_int * max(len(pairs), 1))(*[int(s) for s, _ in pairs])
+        counts = (ctypes.c_longlong * max(len(pairs), 1))(*[int(n) for _, n in pairs])
+        rc = self._lib.spc_reserve_all(self._h, len(pairs), slots, counts)
+        if rc == -1:
+            raise OutOfPages(f"no pages for the step's {sum(n for _, n in pairs)} positions of slots "
+                             f"{[s for s, _ in pairs]}: free {[self.free_pages(g) for g in range(self.n_groups())]}")
+        if rc != 0:
+            raise CacheError("reserve_all: a slot of the step is not live, or named twice")
 
     def commit(self, slot, n):
         rc = self._lib.spc_commit(self._h, slot, n)

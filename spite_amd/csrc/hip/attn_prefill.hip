@@ -223,10 +223,13 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
         // only when some column of the wave needs it (alpha is exactly 1 otherwise)
         const bool rescale = __any(alpha[0] != 1.0f || alpha[1] != 1.0f);
         // keys behind the last query of the wave may lie behind the request's last position, where
-        // the page still holds what its last owner left; a probability of zero times a value that
-        // is not finite is not zero, so those values are taken as zero (the keys below a column's
-        // first visible one are the request's own, and finite)
-        const bool stale = key0 + PF_KEYS - 1 > pq_max;
+        // the page still holds what its last owner left, and a half of the block whose page the
+        // request has given back (the keys below a window's or a chunk's first visible one, where
+        // a page is half a block) was read from a page that is somebody else's or nobody's; a
+        // probability of zero times a value that is not finite is not zero, so those values are
+        // taken as zero (the other keys below a column's first visible one are the request's own,
+        // and finite)
+        const bool stale = key0 + PF_KEYS - 1 > pq_max || absent0 || absent1;
 #pragma unroll
         for (int d = 0; d < ND; ++d) {
             if (rescale) {
@@ -239,7 +242,7 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
                 if (stale) {
 #pragma unroll
                     for (int e = 0; e < 8; ++e)
-                        vf[e] = key0 + hh * 32 + qd * 8 + e > pq_max ? (bf16)0.f : vf[e];
+                        vf[e] = (key0 + hh * 32 + qd * 8 + e > pq_max || (hh ? absent1 : absent0)) ? (bf16)0.f : vf[e];
                 }
 #pragma unroll
                 for (int c = 0; c < 2; ++c)

@@ -23,6 +23,8 @@ enum { SP_F32 = 0, SP_BF16 = 1 };
 // last failure of the calling thread is kept for spite_hip_last_error().
 int sp_fail(const char* fmt, ...);
 #define SP_REQUIRE(cond, ...) do { if (!(cond)) return sp_fail(__VA_ARGS__); } while (0)
+// Compute units of the current device (asked once per device): what tile counts are weighed against.
+int sp_cu_count();
 #define SP_LAUNCH_CHECK(name) do { hipError_t e_ = hipGetLastError(); \
     if (e_ != hipSuccess) return sp_fail("%s: launch failed: %s", name, hipGetErrorString(e_)); } while (0)
 

@@ -12,6 +12,19 @@ int sp_fail(const char* fmt, ...) {
 extern "C" const char* spite_hip_last_error() { return g_err; }
 extern "C" int spite_hip_abi_version() { return 1; }
 
+int sp_cu_count() {
+    static int count[64];                       // per device; 0 = not asked yet
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    int c = __atomic_load_n(&count[dev], __ATOMIC_RELAXED);
+    if (c <= 0) {
+        if (hipDeviceGetAttribute(&c, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || c <= 0) c = 256;
+        __atomic_store_n(&count[dev], c, __ATOMIC_RELAXED);
+    }
+    return c;
+}
+extern "C" int spite_cu_count() { return sp_cu_count(); }
+
 // ------------------------------------------------------------------ embedding
 template <typename T>
 __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table,

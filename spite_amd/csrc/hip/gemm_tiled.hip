@@ -391,15 +391,18 @@ extern "C" int spite_gemm_tiled(const void* X, int ldx, const void* W, long w_gr
     SP_REQUIRE(shape >= 0 && shape <= 6, "gemm_tiled: tile shape %d", shape);
     if (M == 0) return 0;
     if (shape == 0) {
-        // Tiles come in whole numbers per CU: a plain product whose 128-row tiles leave many of the 256
-        // CUs without one (2,048 x 5,120: 160 tiles) takes 96-row tiles when those need no further round
-        // (220 tiles).  A tile's time was measured as 38 + 8.5 us per 16 rows at K = 5,120; the sum over
-        // k runs in the same order in both, so a row's result does not depend on the choice.
+        // Tiles come in whole numbers per CU: a plain product whose 128-row tiles leave many of the
+        // CUs without one (2,048 x 5,120 on 256 CUs: 160 tiles) takes 96-row tiles when those need no
+        // further round (220 tiles).  A tile's time is a fixed part (W's stream, start and end) and a
+        // part per 16 rows, measured as 38 and 8.5 us at K = 5,120 on an MI355X; only their ratio
+        // counts here, and both parts grow with K alike.  The sum over k runs in the same order in
+        // both, so a row's result does not depend on the choice.
+        constexpr double TILE_FIXED = 38.0, TILE_PER_16_ROWS = 8.5;
         shape = 1;
         if (!offsets && !glu) {
-            const long cols = (N + 511) / 512;
-            const long rounds8 = (((M + 127) / 128) * cols + 255) / 256, rounds6 = (((M + 95) / 96) * cols + 255) / 256;
-            if (rounds6 * (38 + 8.5 * 6) < rounds8 * (38 + 8.5 * 8)) shape = 6;
+            const long cus = sp_cu_count(), cols = (N + 511) / 512;
+            const long rounds8 = (((M + 127) / 128) * cols + cus - 1) / cus, rounds6 = (((M + 95) / 96) * cols + cus - 1) / cus;
+            if (rounds6 * (TILE_FIXED + TILE_PER_16_ROWS * 6) < rounds8 * (TILE_FIXED + TILE_PER_16_ROWS * 8)) shape = 6;
         }
     }
     if (shape == 6) {

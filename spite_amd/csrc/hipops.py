@@ -58,6 +58,8 @@ def lib():
             fn = getattr(l, name)
             fn.argtypes = args
             fn.restype = c_int
+        l.spite_cu_count.argtypes = []
+        l.spite_cu_count.restype = c_int
         _lib = l
     return _lib
 
@@ -423,15 +425,27 @@ def operand_order(w: torch.Tensor) -> torch.Tensor:
 
 
 def tiled_k_runs(M: int, N: int, K: int) -> int:
-    """Into how many runs the tiled product cuts its sum over k: with fewer than 128 tiles of
-    128 rows x 512 columns the chip's 256 CUs are not filled, and a run keeps at least four steps
-    of 64 k."""
+    """Into how many runs the tiled product cuts its sum over k: with tiles of 128 rows x 512
+    columns for fewer than half of the chip's CUs, those are not filled, and a run keeps at least
+    four steps of 64 k."""
+    cus = cu_count()
     tiles = -(-M // 128) * -(-N // 512)
     steps = K // 64
-    runs = min(8, 256 // max(tiles, 1), steps // 4)
+    runs = min(8, cus // max(tiles, 1), steps // 4)
     while runs > 1 and -(-steps // runs) * (runs - 1) >= steps:      # no run may be empty
         runs -= 1
-    return runs if tiles < 128 and runs > 1 else 1
+    return runs if tiles < cus // 2 and runs > 1 else 1
+
+
+_cu_count = None
+
+
+def cu_count() -> int:
+    """Compute units of the current GPU, as the library counts them."""
+    global _cu_count
+    if _cu_count is None:
+        _cu_count = int(lib().spite_cu_count())
+    return _cu_count
 
 
 def gemm_tiled(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None, glu=False,

@@ -25,6 +25,7 @@ CacheManager::CacheManager(int page_size, int max_requests, const std::vector<Gr
         s.freed_below.assign(groups_.size(), 0);
     }
     for (int i = max_requests - 1; i >= 0; --i) free_slots_.push_back(i);
+    fresh_.assign(max_requests, 0);
 }
 
 int CacheManager::admit() {
@@ -38,14 +39,18 @@ int CacheManager::admit() {
         sl.table[g].clear();
         sl.freed_below[g] = 0;
     }
-    fresh_.push_back(s);
+    fresh_[s] = 1;
     return s;
 }
 
 int CacheManager::take_fresh(int* out, int cap) {
-    const int n = (int)fresh_.size();
-    for (int i = 0; i < n && i < cap; ++i) out[i] = fresh_[i];
-    fresh_.clear();
+    int n = 0;
+    for (int s = 0; s < (int)fresh_.size(); ++s) {
+        if (!fresh_[s]) continue;
+        if (n < cap) out[n] = s;
+        ++n;
+        fresh_[s] = 0;
+    }
     return n;
 }
 
@@ -89,6 +94,20 @@ int CacheManager::reserve(int slot, int64_t n) {
         }
     }
     sl.reserved = std::max(sl.reserved, sl.cached + n);
+    return 0;
+}
+
+int CacheManager::reserve_all(int n, const int* slots, const int64_t* counts) {
+    std::vector<int64_t> need(groups_.size(), 0);
+    for (int i = 0; i < n; ++i) {
+        if (!live(slots[i]) || counts[i] < 0) return -2;
+        for (int j = 0; j < i; ++j)
+            if (slots[j] == slots[i]) return -2;           // a slot twice: the sums below would be wrong
+        for (int g = 0; g < n_groups(); ++g) need[g] += pages_needed(slots[i], counts[i], g);
+    }
+    for (int g = 0; g < n_groups(); ++g)
+        if (need[g] > free_pages(g)) return -1;
+    for (int i = 0; i < n; ++i) reserve(slots[i], counts[i]);
     return 0;
 }
 

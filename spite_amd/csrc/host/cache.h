@@ -44,10 +44,10 @@ public:
     int free_slots() const { return (int)free_slots_.size(); }
 
     int admit();                               // slot id, or -1 when every slot is taken
-    // Slots handed out since the last call, oldest first (a slot that was admitted, released and
-    // admitted again appears twice): whoever keeps per-request state on the GPU clears the rows
-    // of these slots before the next step runs, whichever caller admitted them.  Returns how
-    // many there were; at most `cap` are written.
+    // Slots handed out since the last call, in ascending order, each once however often it was
+    // admitted and released meanwhile (never more than max_requests): whoever keeps per-request
+    // state on the GPU clears the rows of these slots before the next step runs, whichever
+    // caller admitted them.  Returns how many there were; at most `cap` are written.
     int take_fresh(int* out, int cap);
     bool live(int slot) const;
     int64_t cached(int slot) const;            // positions committed
@@ -57,6 +57,9 @@ public:
     // As can_reserve for a request that is not admitted yet and holds nothing.
     bool can_reserve_new(int64_t n) const;
     int reserve(int slot, int64_t n);          // 0; -1 out of pages (nothing changed); -2 bad slot
+    // reserve() for several slots at once: every one of them gets its pages, or nothing changes
+    // (-1 out of pages, -2 a slot that is not live or named twice).
+    int reserve_all(int n, const int* slots, const int64_t* counts);
     int commit(int slot, int64_t n);           // 0; -2 bad slot; -3 more than was reserved
     int release(int slot);                     // 0; -2 bad slot
     // Pages that a request of `total` positions holds at most at one time in group g, when
@@ -87,7 +90,7 @@ private:
     std::vector<std::vector<int>> free_;       // [group] stack of free pages
     std::vector<Slot> slots_;
     std::vector<int> free_slots_;              // stack, lowest id on top at the start
-    std::vector<int> fresh_;                   // admitted and not yet reported by take_fresh
+    std::vector<char> fresh_;                  // [slot] admitted and not yet reported by take_fresh
 };
 
 }  // namespace spite

@@ -39,6 +39,9 @@ long long spc_cached(void* c, int slot) { return ((CacheManager*)c)->cached(slot
 int spc_can_reserve(void* c, int slot, long long n) { return ((CacheManager*)c)->can_reserve(slot, n); }
 int spc_can_reserve_new(void* c, long long n) { return ((CacheManager*)c)->can_reserve_new(n); }
 int spc_reserve(void* c, int slot, long long n) { return ((CacheManager*)c)->reserve(slot, n); }
+int spc_reserve_all(void* c, int n, const int* slots, const long long* counts) {
+    return ((CacheManager*)c)->reserve_all(n, slots, (const int64_t*)counts);
+}
 int spc_commit(void* c, int slot, long long n) { return ((CacheManager*)c)->commit(slot, n); }
 int spc_release(void* c, int slot) { return ((CacheManager*)c)->release(slot); }
 int spc_free_pages(void* c, int g) { return ((CacheManager*)c)->free_pages(g); }

@@ -28,6 +28,7 @@ def lib():
             "spc_can_reserve": (I, [P, I, LL]),
             "spc_can_reserve_new": (I, [P, LL]),
             "spc_reserve": (I, [P, I, LL]),
+            "spc_reserve_all": (I, [P, I, PI, PLL]),
             "spc_commit": (I, [P, I, LL]),
             "spc_release": (I, [P, I]),
             "spc_free_pages": (I, [P, I]),

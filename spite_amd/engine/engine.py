@@ -78,6 +78,10 @@ class StepMeta:
         for name, sz in sizes:
             offs[name] = (total, sz)
             total += (sz + 63) // 64 * 64
+        # where every array lies in the buffer: a captured step holds these addresses, so a step
+        # may replay a graph only if its layout is the same (a part's derived array may change
+        # its size between two steps of one shape)
+        self.layout = tuple(o for o, _ in offs.values())
         host = engine._pinned(total)
         hv = {name: host[o:o + sz] for name, (o, sz) in offs.items()}
         tok = hv["token_ids"]
@@ -247,8 +251,7 @@ class Engine:
                 raise EngineError(f"entry {i}: token id {bad} outside the vocabulary of {V}")
             total += len(e.tokens)
         self.cache.zero_fresh()       # state rows of slots handed out since the last step, by whomever
-        for e in entries:
-            self.cache.reserve(e.slot, len(e.tokens))
+        self.cache.reserve_all([(e.slot, len(e.tokens)) for e in entries])    # every entry's pages, or nothing
         meta = StepMeta(self, entries)
         if trace is not None:
             meta.ctx.extras["trace"] = trace
@@ -256,7 +259,7 @@ class Engine:
         key = None
         if (self.use_graphs and trace is None and meta.ctx.decode_only and meta.ctx.n_out == meta.ctx.n_seqs
                 and all(tuple(e.want) == (0,) for e in entries)):
-            key = (meta.ctx.n_seqs, meta.widths)
+            key = (meta.ctx.n_seqs, meta.widths, meta.layout)
             logits = self._replay(key, meta)
         if logits is None:
             self._step_ws.reset()

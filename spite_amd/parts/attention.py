@@ -98,15 +98,15 @@ class Attention(Mixer):
     def _decode(self, q, o, ctx, cache, T):
         """The split-KV kernel over the step's first T tokens, each the only one of its request."""
         H, G, hd = self.H, self.G, self.hd
-        # split the keys so that about five hundred workgroups run (measured: more splits only
-        # add partial results to combine), each with at least eight blocks of keys; the
+        # split the keys so that about two workgroups a compute unit run (measured: more splits
+        # only add partial results to combine), each with at least eight blocks of keys; the
         # bound on the keys is the block table's width, so the launch is the same for every
         # step of that shape
         longest = cache.block_table.shape[1] * cache.page_size
         if self.visibility != "full":
             longest = min(longest, self.span + 32)
         blocks = -(-longest // 32)
-        n_splits = max(1, min(-(-512 // (T * G)), -(-blocks // 8), 256))
+        n_splits = max(1, min(-(-2 * hipops.cu_count() // (T * G)), -(-blocks // 8), 256))
         scratch = ctx.ws.take((hipops.attn_decode_workspace(T, H, hd, n_splits) // 4,), torch.float32)
         hipops.attn_decode(q, cache.k_pages, cache.v_pages, o, scratch, ctx.positions, ctx.seq_of_token,
                            cache.block_table, T, H, G, hd, cache.page_size, self.visibility, self.span,

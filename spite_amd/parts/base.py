@@ -203,7 +203,10 @@ def register_step_array(name: str, fn: Callable) -> None:
     want on the GPU.  It is computed only for models in which a part lists ``name`` in its
     ``step_arrays``, travels in the step's one metadata copy, and is found under
     ``ctx.derived[name]`` as ``(device array, info)``; ``info`` is any host-side fact that goes
-    with it.  The function must depend on its argument alone."""
+    with it.  The function must depend on its argument alone.  A captured decode step is
+    replayed only for steps whose metadata lies at the same places in the step's buffer, so an
+    array whose size changes between two decode steps of one shape costs a new capture each time
+    it does: keep its size a function of the step's shape (entries and their token counts)."""
     _STEP_ARRAYS[name] = fn
 
 

@@ -158,11 +158,13 @@ def random_tensors(config: dict, seed: int, std: float = 0.02, device=None) -> D
 
 
 def write_random_model(folder: str, config: dict, seed: int, std: float = 0.02, dtype: str | None = None,
-                       overrides: Dict[str, torch.Tensor] | None = None, device=None) -> str:
+                       overrides: Dict[str, torch.Tensor] | None = None, device=None, keep_wide=()) -> str:
     """Writes ``folder/config.json`` and ``folder/model.safetensors``; returns the folder.
 
     ``dtype`` of the stored matrices defaults to the config's ``torch_dtype``.  ``overrides``
-    replaces tensors by name (tests plant special weights this way)."""
+    replaces tensors by name (tests plant special weights this way).  ``keep_wide``: substrings of
+    tensor names that are stored in float32 whatever ``dtype`` is (a checkpoint that keeps some
+    of its tensors in 32-bit beside bfloat16 ones)."""
     config = dict(config)
     dtype = dtype or config.get("torch_dtype", "bfloat16")
     if dtype not in _FILE_DTYPES:
@@ -175,7 +177,9 @@ def write_random_model(folder: str, config: dict, seed: int, std: float = 0.02, 
         if tuple(t.shape) != tuple(tensors[name].shape):
             raise ValueError(f"override for {name}: shape {tuple(t.shape)}, expected {tuple(tensors[name].shape)}")
         tensors[name] = t.to(torch.float32) if t.is_floating_point() else t
-    stored = {n: (t.to(_FILE_DTYPES[dtype]) if t.is_floating_point() else t) for n, t in tensors.items()}
+    wide = lambda n: any(k in n for k in keep_wide)
+    stored = {n: (t.to(torch.float32 if wide(n) else _FILE_DTYPES[dtype]) if t.is_floating_point() else t)
+              for n, t in tensors.items()}
     os.makedirs(folder, exist_ok=True)
     config["spite_random_init"] = {"seed": int(seed), "std": float(std), "matrices": "N(0,std)",
                                    "norm_weights": "1+N(0,std)"}

@@ -41,7 +41,14 @@ TINY_C = dict(
     rope_theta=50000.0, rope_scaling=None, attention_chunk_size=64, no_rope_layers=[1, 0, 1, 1],
     use_qk_norm=True, attn_temperature_tuning=True, floor_scale=32, attn_scale=0.2,
     tie_word_embeddings=False, torch_dtype="float32")
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+# the reference's own reading of the rotating layers: the last `attention_chunk_size` keys
+# (crates/spite-models/src/llama/llama4.rs:189-197) instead of the chunk
+TINY_BW = dict(TINY_B, attention_local_kind="window")
+TINY_CW = dict(TINY_C, attention_local_kind="window", attention_chunk_size=100)
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "Bw": TINY_BW, "Cw": TINY_CW, "Cm": TINY_C}
+# "Cm": a bfloat16 folder of C whose shared experts are stored in 32-bit: the engine keeps them so,
+# and the shared expert cannot be one more group of the experts' bfloat16 products
+KEEP_WIDE = {"Cm": ("shared_expert",)}
 
 
 def planted_tensors(cfg: dict, seed: int, std: float = 0.05, qk_gain: float = 2.0, router_gain: float = 8.0):
@@ -59,11 +66,11 @@ def planted_tensors(cfg: dict, seed: int, std: float = 0.05, qk_gain: float = 2.
     return t
 
 
-def make_model(folder: str, cfg: dict, seed: int = 1, dtype: str = "float32", **kw) -> dict:
+def make_model(folder: str, cfg: dict, seed: int = 1, dtype: str = "float32", keep_wide=(), **kw) -> dict:
     """Writes a model folder; returns the weights as the file holds them (after rounding to
     the file's dtype), widened to float64, for the plain implementation."""
     from spite_amd.weights.random_init import write_random_model
-    write_random_model(folder, cfg, seed, dtype=dtype, overrides=planted_tensors(cfg, seed, **kw))
+    write_random_model(folder, cfg, seed, dtype=dtype, overrides=planted_tensors(cfg, seed, **kw), keep_wide=keep_wide)
     return read_weights(folder)
 
 

@@ -86,6 +86,21 @@ def test_pages_that_are_given_back_are_handed_out_next():
     c.check()
 
 
+def test_a_step_gets_all_its_pages_or_none():
+    c = make([CHUNK32, FULL], 16, 5)
+    a, b, d = c.admit(), c.admit(), c.admit()
+    c.reserve_all([(a, 20), (b, 16)])                       # 2 + 1 pages of either group
+    assert c.free_pages(0) == 2 and c.free_pages(1) == 2
+    with pytest.raises(OutOfPages):                         # a: none more, b: one more, d: two: three in all
+        c.reserve_all([(a, 30), (b, 17), (d, 20)])
+    assert c.free_pages(0) == 2 and len(c.block_table(b, 0)) == 1 and c.block_table(d, 0) == []
+    c.reserve_all([(a, 30), (b, 17), (d, 16)])              # one for b, one for d
+    assert c.free_pages(0) == 0 and c.free_pages(1) == 0
+    with pytest.raises(CacheError):
+        c.reserve_all([(a, 1), (a, 1)])
+    c.check()
+
+
 def test_running_out_changes_nothing():
     c = make([CHUNK32, FULL], 16, 3)
     s = c.admit()
@@ -199,6 +214,26 @@ def test_slots_handed_out_are_reported_once_whoever_admitted_them():
     # released and admitted again between two steps: reported, once
     c.release(s)
     assert c.admit() == s and c.states[0][s].abs().sum() == 0
+
+
+def test_a_storm_of_admissions_clears_no_running_request():
+    # many admissions and releases between two steps: every slot that changed hands is reported
+    # once, and the state of a request that kept running meanwhile is not touched
+    need = CacheNeed(kv=KVNeed(1, 16, "full"), state=StateNeed((3,), torch.float32))
+    c = PagedCache([need], 16, 8, 3, torch.float32, torch.device("cpu"))
+    runner = c.admit()
+    assert c.zero_fresh() == []
+    c.states[0][runner] = 5.0
+    lib, h = c._lib, c._h
+    for _ in range(200):                                     # behind the Python object's back, as a scheduler would
+        s = lib.spc_admit(h)
+        assert s >= 0 and s != runner
+        lib.spc_release(h, s)
+    s = lib.spc_admit(h)
+    c.states[0][s] = 9.0
+    got = c.zero_fresh()
+    assert s in got and runner not in got and len(got) == len(set(got)) <= 2
+    assert c.states[0][runner].tolist() == [5.0] * 3 and c.states[0][s].abs().sum() == 0
 
 
 def test_a_chunked_group_gets_no_more_pages_than_its_requests_can_hold():

@@ -542,6 +542,10 @@ PORTION_CASES = [
     (2, 2, 64, 32, [600, 3], [(0, 100, 500), (1, 0, 3)], "full", 0),           # one head a kv head: tiles of 256
     (40, 8, 128, 64, [700], [(0, 300, 400)], "window", 257),
     (34, 2, 64, 96, [400], [(0, 0, 400)], "full", 0),                          # 17 heads a kv head, pages of 96
+    # the first visible key (96) lies on a page with an odd index: the block of 64 keys that holds it
+    # begins on a page that was given back
+    (16, 1, 64, 32, [500], [(0, 195, 120)], "window", 100),
+    (10, 2, 128, 32, [400, 50], [(0, 230, 90), (1, 10, 40)], "chunk", 96),
 ]
 
 
@@ -557,6 +561,12 @@ def test_attn_prefill(case, key_split):
     qs = torch.randn(T, H, hd, generator=g).to(dtype)
     for s, first, count in portions:
         kv.drop_below(s, plain_first(vis, span, first))
+    # pages that no request holds (given back, or never handed out) are somebody else's: nothing of
+    # them may reach the output, not even through a probability of zero
+    held = {int(p) for p in kv.bt.flatten().tolist() if p >= 0}
+    for p in range(kv.kp.shape[0]):
+        if p not in held:
+            kv.kp[p], kv.vp[p] = float("nan"), float("nan")
     ref = attention_reference(kv, queries, qs, H, vis, span)
     positions = torch.tensor([p for _, p in queries], dtype=torch.int32, device=DEV)
     seq = torch.tensor([i for i, (s, first, count) in enumerate(portions) for _ in range(count)], dtype=torch.int32, device=DEV)
@@ -880,5 +890,14 @@ def test_mfma_loop_runs_and_counts_its_flops():
     flops = ops().mfma_loop(out, 10, 0.0)
     torch.cuda.synchronize()
     assert flops == 8 * 8 * 10 * 32 * 16384 and float(out.abs().sum()) == 0.0
-    ops().mfma_loop(out, 10, 1.0)
-    assert torch.isfinite(out).all() and float(out.abs().sum()) > 0.0
+    # the sums are the loop's work: twice the steps give twice the sums (the same products are
+    # added again), operands of half the size a quarter (exactly: a power of two); a loop that
+    # dropped or repeated products would break the first, one that ignored its operands the second
+    def sums(steps, gain):
+        ops().mfma_loop(out, steps, gain)
+        torch.cuda.synchronize()
+        return out.double().cpu()
+    one, two, half = sums(10, 1.0), sums(20, 1.0), sums(10, 0.5)
+    assert torch.isfinite(one).all() and float(one.abs().max()) > 0.0 and one.unique().numel() > 1
+    assert float((two - 2 * one).abs().max()) <= 1e-4 * float(one.abs().max())
+    assert torch.equal(half * 4, one)

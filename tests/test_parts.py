@@ -203,6 +203,45 @@ def test_experts_with_weights_in_operand_order(T):
     assert err <= 1e-2 * ref.abs().max().item(), (T, err, ref.abs().max().item())
 
 
+@pytest.mark.parametrize("T", [7, 40, 150])
+@pytest.mark.parametrize("how", ["shared expert of another width", "shared expert kept in 32-bit"])
+def test_experts_with_a_shared_expert_of_its_own(T, how):
+    """The experts' part when the shared expert cannot be one more group of the grouped products:
+    its intermediate size differs from the routed experts', or the checkpoint kept it in 32-bit
+    beside bfloat16 experts.  It then runs as two plain products of its own."""
+    from spite_amd.engine.context import Env, Workspace, StepContext, HostBatch
+    from spite_amd.parts.feed_forward import MoeTop1Sigmoid
+    d, F_, E = 128, 64, 8
+    Fs = 96 if how == "shared expert of another width" else F_
+    wide = how == "shared expert kept in 32-bit"
+    g = torch.Generator().manual_seed(200 + T)
+    rnd = lambda *s, std=1.0: torch.randn(*s, generator=g) * std
+    w = {"router": rnd(E, d, std=0.5), "experts.gate_up_proj": rnd(E, d, 2 * F_, std=0.1),
+         "experts.down_proj": rnd(E, F_, d, std=0.1), "shared.gate_proj": rnd(Fs, d, std=0.1),
+         "shared.up_proj": rnd(Fs, d, std=0.1), "shared.down_proj": rnd(d, Fs, std=0.1)}
+    w = {k: (v if k == "router" or (wide and k.startswith("shared.")) else v.to(torch.bfloat16)) for k, v in w.items()}
+    part = MoeTop1Sigmoid(Env(torch.bfloat16, torch.device(DEV)), hidden_size=d, intermediate_size=F_, n_experts=E,
+                          shared_intermediate_size=Fs)
+    part.load({k: v.to(DEV) for k, v in w.items()})
+    assert not part.fused_shared and part.ws_gate_up is not None
+    assert part.ws_gate_up.dtype == (torch.float32 if wide else torch.bfloat16)
+    x = rnd(T, d).to(torch.bfloat16)
+    ctx = StepContext(T=T, n_seqs=1, token_ids=None, positions=None, seq_of_token=None, cu_seqlens=None,
+                      seq_slots=None, seq_starts=None, logit_rows=None, n_out=0,
+                      host=HostBatch(np.zeros(1), np.zeros(1), np.full(1, T), np.array([0, T])),
+                      ws=Workspace(torch.device(DEV), 1 << 24))
+    outs = part.forward(x.to(DEV), x.to(DEV).float(), ctx)
+    W = {k: v.double() for k, v in w.items()}
+    ref = plain.moe_ffn(x.double(), W["router"], W["experts.gate_up_proj"], W["experts.down_proj"],
+                        W["shared.gate_proj"], W["shared.up_proj"], W["shared.down_proj"])
+    got = sum(o.double() for o in outs).cpu()
+    err = (got - ref).abs().max().item()
+    assert err <= 1e-2 * ref.abs().max().item(), (T, how, err, ref.abs().max().item())
+    # the shared expert's share alone, so that a shared expert that never ran cannot hide behind the routed one
+    alone = plain.swiglu_mlp(x.double(), W["shared.gate_proj"], W["shared.up_proj"], W["shared.down_proj"])
+    assert (outs[1].double().cpu() - alone).abs().max().item() <= 1e-2 * alone.abs().max().item()
+
+
 def test_block_alone(rig):
     from spite_amd.parts.base import LayerCall
     cfg, W = rig.cfg, rig.w

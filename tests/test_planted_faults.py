@@ -17,7 +17,10 @@ import helpers as H
 
 pytestmark = pytest.mark.gpu
 
-CASES = [("A", "float32", 16), ("B", "float32", 8), ("C", "bfloat16", 32), ("C", "float32", 32)]
+# "Cw": a window of 100 keys over pages of 32: the first visible key's page has an odd index at
+# times, so that a block of 64 keys begins on a page that the request has already given back
+CASES = [("A", "float32", 16), ("B", "float32", 8), ("C", "bfloat16", 32), ("C", "float32", 32),
+         ("Cw", "bfloat16", 32), ("Bw", "float32", 8)]
 
 
 def steps_for(cfg):

@@ -82,7 +82,7 @@ def test_bfloat16_against_32_bit_at_the_layer_sizes_of_scout(tmp_path):
           f"relative error of a token's logits: median {np.median(list(errs.values())):.3e}, worst {errs[worst]:.3e} at {worst}")
     top = sorted(errs, key=errs.get, reverse=True)[:8]
     print("[scout sizes] worst tokens:", [(k, round(errs[k], 4)) for k in top])
-    assert others <= 0.1 * n_tok
+    assert others <= 0.03 * n_tok, (others, n_tok)
     # A logit passes some twenty-five roundings to bfloat16 (q, k, v, the probabilities, the
     # attention's output, the normed rows, the experts' activations, in two layers, and the last
     # normed row), each an independent relative error of about 2^-9 to 2^-8 of what it rounds:

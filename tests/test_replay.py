@@ -32,7 +32,8 @@ REQUESTS = {
     "B": {"b0": 1 + 16, "b1": 7 + 16, "b2": 16 + 16, "b3": 33 + 16, "b4": 70 + 16},
     "C": {"c0": 5 + 16, "c1": 70, "c2": 150, "c3": 300},
 }
-PAGE = {"A": 16, "B": 8, "C": 32}
+REQUESTS.update({"Bw": REQUESTS["B"], "Cw": REQUESTS["C"], "Cm": REQUESTS["C"]})
+PAGE = {"A": 16, "B": 8, "C": 32, "Bw": 8, "Cw": 32, "Cm": 32}
 
 
 class Case:
@@ -40,7 +41,7 @@ class Case:
         from spite_amd.engine.engine import Engine
         self.name, self.dtype, self.cfg = name, dtype, H.CONFIGS[name]
         self.dir = str(tmp / f"{name}_{dtype}")
-        self.weights = H.make_model(self.dir, self.cfg, seed=7, dtype=dtype)
+        self.weights = H.make_model(self.dir, self.cfg, seed=7, dtype=dtype, keep_wide=H.KEEP_WIDE.get(name, ()))
         self.reqs = {rid: H.random_tokens(self.cfg["vocab_size"], n, 100 + i)
                      for i, (rid, n) in enumerate(REQUESTS[name].items())}
         self.plain = H.plain_logits(self.cfg, self.weights, self.reqs)
@@ -78,7 +79,8 @@ class Case:
         return ref
 
 
-@pytest.fixture(scope="module", params=[("A", "float32"), ("B", "float32"), ("A", "bfloat16"), ("B", "bfloat16"), ("C", "bfloat16")],
+@pytest.fixture(scope="module", params=[("A", "float32"), ("B", "float32"), ("A", "bfloat16"), ("B", "bfloat16"), ("C", "bfloat16"),
+                                        ("Bw", "float32"), ("Bw", "bfloat16"), ("Cw", "bfloat16"), ("Cm", "bfloat16")],
                 ids=lambda p: f"{p[0]}-{p[1]}")
 def case(request, tmp_path_factory):
     return Case(*request.param, tmp_path_factory.mktemp("replay"))
@@ -270,10 +272,11 @@ def test_faults_are_visible(case):
     the reference's sliding window in place of chunks, or with one expert swapped, differs
     from the right logits by far more than the tolerance."""
     import plain_llama4 as plain
-    rid = {"A": "a3", "B": "b4", "C": "c3"}[case.name]
+    rid = {"A": "a3", "B": "b4", "C": "c3"}[case.name[0]]
     toks = case.reqs[rid]
     right = np.stack([case.plain[(rid, i)] for i in range(len(toks))])
-    window = plain.forward(case.cfg, case.weights, toks, visibility="window").numpy()
+    other = "chunk" if case.cfg.get("attention_local_kind") == "window" else "window"
+    window = plain.forward(case.cfg, case.weights, toks, visibility=other).numpy()
     assert np.abs(window - right).max() > 3 * case.tol
     w2 = dict(case.weights)
     moe_layer = 1

@@ -41,18 +41,32 @@ def _both(lib, T, H, G, hd, ps, ctx_len, n_splits, vis, span, seed):
     torch.cuda.synchronize()
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     P = ctypes.c_void_p
-    before = torch.cuda.memory_allocated()
-    rc = lib.spite_attn_decode_static(
+    call = lambda: lib.spite_attn_decode_static(
         P(q.data_ptr()), P(kp.data_ptr()), P(vp.data_ptr()), P(out_st.data_ptr()), P(positions.data_ptr()),
         P(seq.data_ptr()), P(bt.data_ptr()), ctypes.c_int(bt.shape[1]), ctypes.c_int(T), ctypes.c_int(H),
         ctypes.c_int(G), ctypes.c_int(hd), ctypes.c_int(ps), ctypes.c_int(hipops.VIS[vis]), ctypes.c_int(span),
         ctypes.c_float(hd ** -0.5), ctypes.c_int(n_splits), stream)
+    if not _both.warm:
+        # the process's first call looks the array's address up (and the runtime may set up what a
+        # first launch of these kernels needs); what is measured is a call after that
+        assert call() == 0, lib.spite_hip_last_error().decode()
+        torch.cuda.synchronize()
+        _both.warm = True
+        out_st.fill_(7.0)
+        torch.cuda.synchronize()
+    # free device memory as the driver counts it: an allocation inside the library, which torch's
+    # own counters would not see, shows here
+    before = torch.cuda.mem_get_info()[0]
+    rc = call()
     assert rc == 0, lib.spite_hip_last_error().decode()
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == before
     assert torch.isfinite(out_st.float()).all()
     assert torch.equal(out_ws, out_st), (out_ws.float() - out_st.float()).abs().max()
     return out_st
+
+
+_both.warm = False
 
 
 def test_static_scratch_matches_the_workspace_form_twice_in_a_row():
