@@ -218,6 +218,18 @@ void attn_decode_combine_kernel(const float* __restrict__ part, bf16* __restrict
     out[((size_t)t * H + h) * HD + c] = (bf16)(acc * linv);
 }
 
+// Joins the splits' records [T][H][n_splits][hd + 2] (output not yet divided, maximum, sum) into
+// the bf16 output [T][H][hd]; the prefill kernel's splits leave the same records.
+int sp_attn_combine(const float* part, void* out, int T, int H, int hd, int n_splits, hipStream_t st) {
+    SP_REQUIRE(T >= 0 && H > 0 && H <= 65535 && n_splits >= 1 && n_splits <= 256 && (hd == 64 || hd == 128),
+               "attn_combine: T=%d H=%d hd=%d splits=%d", T, H, hd, n_splits);
+    if (T == 0) return 0;
+    if (hd == 128) attn_decode_combine_kernel<128><<<dim3(T, H), 128, 0, st>>>(part, (bf16*)out, H, n_splits);
+    else attn_decode_combine_kernel<64><<<dim3(T, H), 64, 0, st>>>(part, (bf16*)out, H, n_splits);
+    SP_LAUNCH_CHECK("attn_combine");
+    return 0;
+}
+
 // Bytes of fp32 scratch that a call needs.
 extern "C" size_t spite_attn_decode_workspace(int T, int H, int hd, int n_splits) {
     return (size_t)T * H * n_splits * (hd + 2) * sizeof(float);

@@ -25,6 +25,8 @@ int sp_fail(const char* fmt, ...);
 #define SP_REQUIRE(cond, ...) do { if (!(cond)) return sp_fail(__VA_ARGS__); } while (0)
 // Compute units of the current device (asked once per device): what tile counts are weighed against.
 int sp_cu_count();
+// attn_decode.hip: joins the records that split attention leaves (see there).
+int sp_attn_combine(const float* part, void* out, int T, int H, int hd, int n_splits, hipStream_t st);
 #define SP_LAUNCH_CHECK(name) do { hipError_t e_ = hipGetLastError(); \
     if (e_ != hipSuccess) return sp_fail("%s: launch failed: %s", name, hipGetErrorString(e_)); } while (0)
 

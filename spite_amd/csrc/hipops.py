@@ -49,7 +49,8 @@ def lib():
             "spite_gemm_mfma": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, P],
             "spite_gemm_tiled": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, P],
             "spite_gemm_tiled_split": [P, I, P, P, I, I, I, I, I, I, P, P],
-            "spite_attn_prefill": [P, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, F, F, I, P],
+            "spite_attn_prefill": [P, P, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, F, F, P, I, P],
+            "spite_attn_prefill_splits": [P, I, I, I, L],
             "spite_argmax_rows": [P, I, I, I, P, P, P, P],
             "spite_stream_read": [P, c_size_t, P, I, P],
             "spite_mfma_loop": [P, I, I, F, P],
@@ -58,6 +59,8 @@ def lib():
             fn = getattr(l, name)
             fn.argtypes = args
             fn.restype = c_int
+        l.spite_attn_prefill_workspace.argtypes = [P, I, I, I, I, I]
+        l.spite_attn_prefill_workspace.restype = c_size_t
         l.spite_cu_count.argtypes = []
         l.spite_cu_count.restype = c_int
         _lib = l
@@ -475,12 +478,29 @@ def gemm_tiled(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_sca
         int(shape), _stream()), "gemm_tiled")
 
 
+def attn_prefill_splits(counts, H, G, max_keys) -> int:
+    """Into how many splits the prefill kernel's tiles of this step are best cut (1: none), for
+    ``counts`` query tokens per request and at most ``max_keys`` keys read by a query."""
+    counts = np.ascontiguousarray(counts, dtype=np.int32)
+    return int(lib().spite_attn_prefill_splits(counts.ctypes.data, int(counts.size), H, G, int(max_keys)))
+
+
+def attn_prefill_workspace(counts, H, G, hd, n_splits) -> int:
+    """Bytes of fp32 scratch that ``attn_prefill`` needs for ``n_splits`` > 1 (none for 1)."""
+    counts = np.ascontiguousarray(counts, dtype=np.int32)
+    return int(lib().spite_attn_prefill_workspace(counts.ctypes.data, int(counts.size), H, G, hd, int(n_splits)))
+
+
 def attn_prefill(q, k_pages, v_pages, out, positions, cu_seqlens, counts, block_table,
-                 H, G, hd, page_size, vis, span, scale, key_split=0, softcap=0.0):
+                 H, G, hd, page_size, vis, span, scale, n_splits=1, scratch=None, softcap=0.0, slopes=None):
     """Prefill attention on MFMA (bf16; head sizes 64 and 128; pages of a multiple of 32 keys, in
     operand order).
     ``counts``: the number of query tokens of every request of the step, on the host, in the
-    order of ``cu_seqlens`` (their running sum, on the device) and of the block table's rows."""
+    order of ``cu_seqlens`` (their running sum, on the device) and of the block table's rows.
+    ``n_splits`` > 1 deals every tile's keys to that many workgroups; ``scratch`` (fp32,
+    ``attn_prefill_workspace`` bytes) then holds their partial results.
+    ``slopes`` (fp32 [H] or None): a bias slopes[head] * (key position - query position) on the
+    scaled scores, before the cap."""
     if q.dtype != torch.bfloat16:
         raise KernelError(f"attn_prefill: bfloat16 only, got {q.dtype}")
     counts = np.ascontiguousarray(counts, dtype=np.int32)
@@ -493,13 +513,25 @@ def attn_prefill(q, k_pages, v_pages, out, positions, cu_seqlens, counts, block_
         raise KernelError("attn_prefill: metadata too small")
     if cu_seqlens.numel() < n_seqs + 1:
         raise KernelError("attn_prefill: cu_seqlens shorter than the requests of the step")
+    n_splits = int(n_splits)
+    if n_splits > 1 and (scratch is None or scratch.numel() * 4 < attn_prefill_workspace(counts, H, G, hd, n_splits)):
+        raise KernelError(f"attn_prefill: {n_splits} splits need {attn_prefill_workspace(counts, H, G, hd, n_splits)} bytes of scratch")
     dt = torch.bfloat16
     _check(lib().spite_attn_prefill(
         _ptr(q, "q", dt), _ptr(k_pages, "k_pages", dt), _ptr(v_pages, "v_pages", dt), _ptr(out, "out", dt),
+        _ptr(scratch, "scratch", torch.float32) if n_splits > 1 else None,
         _ptr(positions, "positions", torch.int32), _ptr(cu_seqlens, "cu_seqlens", torch.int32),
         counts.ctypes.data, n_seqs, _ptr(block_table, "block_table", torch.int32), block_table.shape[1],
-        H, G, hd, page_size, VIS[vis], int(span or 0), float(scale), float(softcap), int(key_split), _stream()),
-        "attn_prefill")
+        H, G, hd, page_size, VIS[vis], int(span or 0), float(scale), float(softcap), _slopes(slopes, H), n_splits,
+        _stream()), "attn_prefill")
+
+
+def _slopes(slopes, H):
+    if slopes is None:
+        return None
+    if slopes.numel() != H:
+        raise KernelError(f"score slopes: {slopes.numel()} values for {H} query heads")
+    return _ptr(slopes, "slopes", torch.float32)
 
 
 def argmax_rows(logits, out, scratch_v, scratch_i, n_rows=None):

@@ -112,6 +112,23 @@ class Attention(Mixer):
                            cache.block_table, T, H, G, hd, cache.page_size, self.visibility, self.span,
                            self.scale, n_splits, softcap=self.score_cap)
 
+    def _prefill(self, q, o, ctx, cache, lead, cu_seqlens):
+        """The tiled kernel over the step's entries from ``lead`` on (portions of prompts)."""
+        H, G, hd = self.H, self.G, self.hd
+        counts, starts = ctx.host.counts[lead:], ctx.host.starts[lead:]
+        # the most keys that a query of the step reads: what its request has cached, or no more than
+        # the layer's span and the portion
+        longest = int((starts + counts).max())
+        if self.visibility != "full":
+            longest = min(longest, self.span + int(counts.max()))
+        n_splits = hipops.attn_prefill_splits(counts, H, G, longest)
+        scratch = None
+        if n_splits > 1:
+            scratch = ctx.ws.take((hipops.attn_prefill_workspace(counts, H, G, hd, n_splits) // 4,), torch.float32)
+        hipops.attn_prefill(q, cache.k_pages, cache.v_pages, o, ctx.positions[lead:], cu_seqlens, counts,
+                            cache.block_table[lead:], H, G, hd, cache.page_size, self.visibility, self.span, self.scale,
+                            n_splits=n_splits, scratch=scratch, softcap=self.score_cap)
+
     def forward(self, x, ctx, cache):
         T = x.shape[0]
         H, G, hd = self.H, self.G, self.hd
@@ -140,13 +157,9 @@ class Attention(Mixer):
             if lead and H // G <= 16:
                 # decoded tokens of other requests beside prompt portions
                 self._decode(q, o, ctx, cache, lead)
-                hipops.attn_prefill(q[lead:], cache.k_pages, cache.v_pages, o[lead:], ctx.positions[lead:], cu_tail,
-                                    ctx.host.counts[lead:], cache.block_table[lead:], H, G, hd, cache.page_size,
-                                    self.visibility, self.span, self.scale, softcap=self.score_cap)
             else:
-                hipops.attn_prefill(q, cache.k_pages, cache.v_pages, o, ctx.positions, ctx.cu_seqlens, ctx.host.counts,
-                                    cache.block_table, H, G, hd, cache.page_size, self.visibility, self.span, self.scale,
-                                    softcap=self.score_cap)
+                lead = 0
+            self._prefill(q[lead:], o[lead:], ctx, cache, lead, cu_tail if lead else ctx.cu_seqlens)
         else:
             hipops.attn_generic(q, cache.k_pages, cache.v_pages, o, ctx.positions, ctx.seq_of_token,
                                 cache.block_table, T, H, G, hd, cache.page_size, self.visibility, self.span,

@@ -542,6 +542,7 @@ PORTION_CASES = [
     (2, 2, 64, 32, [600, 3], [(0, 100, 500), (1, 0, 3)], "full", 0),           # one head a kv head: tiles of 256
     (40, 8, 128, 64, [700], [(0, 300, 400)], "window", 257),
     (34, 2, 64, 96, [400], [(0, 0, 400)], "full", 0),                          # 17 heads a kv head, pages of 96
+    (40, 1, 64, 32, [333, 9], [(0, 280, 53), (1, 0, 9)], "chunk", 160),          # 40 heads a kv head: a wave's columns are one query's
     # the first visible key (96) lies on a page with an odd index: the block of 64 keys that holds it
     # begins on a page that was given back
     (16, 1, 64, 32, [500], [(0, 195, 120)], "window", 100),
@@ -549,9 +550,9 @@ PORTION_CASES = [
 ]
 
 
-@pytest.mark.parametrize("key_split", [1, 2])
+@pytest.mark.parametrize("n_splits", [1, 2, 5])
 @pytest.mark.parametrize("case", PORTION_CASES, ids=lambda c: f"H{c[0]}G{c[1]}hd{c[2]}ps{c[3]}{c[6]}")
-def test_attn_prefill(case, key_split):
+def test_attn_prefill(case, n_splits):
     H, G, hd, ps, lens, portions, vis, span = case
     dtype = torch.bfloat16
     kv = PagedKV(lens, G, hd, ps, dtype, seed=3)
@@ -577,7 +578,9 @@ def test_attn_prefill(case, key_split):
     out = torch.zeros(T, H * hd, dtype=dtype, device=DEV)
     ops().attn_prefill(qs.reshape(T, H * hd).to(DEV), *ops().kv_operand_order(kv.kp.to(DEV), kv.vp.to(DEV)), out, positions,
                        torch.tensor(cu, dtype=torch.int32, device=DEV), [count for _, _, count in portions], bt,
-                       H, G, hd, ps, vis, span, 1.0 / math.sqrt(hd), key_split=key_split)
+                       H, G, hd, ps, vis, span, 1.0 / math.sqrt(hd), n_splits=n_splits,
+                       scratch=torch.full((ops().attn_prefill_workspace([c for _, _, c in portions], H, G, hd, n_splits) // 4 + 1,),
+                                          float("nan"), device=DEV))
     got = out.double().cpu().view(T, H, hd)
     assert torch.isfinite(got).all()
     assert (got - ref).abs().max() < 1.5e-2 * max(1.0, float(ref.abs().max()))
