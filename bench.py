@@ -20,8 +20,11 @@ scheduler in portions of 2,048 (pages roll off behind the chunk of 8,192 on the 
 layers), then 64 decoded tokens each, through ``Engine.generate``.
 ``serve``: 12 layers with 128 experts in every second layer, 32 requests with prompts of 512
 to 2,048 tokens, 64 new tokens each: decoded tokens lead prompt portions in mixed steps.
-Both report prefill and decode tokens a second, time to first token, step-time percentiles
-and the most pages held per group of layers.
+Both run three times (``--runs``) and report the median repetition: prefill and decode tokens
+a second, the decode steps against the bytes they have to read, time to first token,
+step-time percentiles and the most pages held per group of layers; ``longctx`` then decodes 64
+tokens with all of its requests live at the prompt's length.  The default run carries both,
+shortened, under ``workloads`` (``--no-workloads`` leaves them out).
 """
 import argparse
 import json
@@ -85,6 +88,12 @@ class Sizes:
         return (self.L * (self.proj * it + 2 * c.hidden_size * 4) + moe_bytes + (self.L - self.n_moe) * self.dense * it
                 + batch * self.seen(context) * self.kv_token + c.vocab_size * c.hidden_size * it
                 + batch * c.hidden_size * it + c.hidden_size * 4)
+
+    def decode_bytes_at(self, contexts, experts_touched):
+        """As ``decode_bytes`` for requests at positions of their own."""
+        b = len(contexts)
+        return self.decode_bytes(b, 0, experts_touched) - b * self.seen(0) * self.kv_token \
+            + sum(self.seen(c) for c in contexts) * self.kv_token
 
     def pairs(self, T, past):
         full = T * past + T * (T + 1) // 2
@@ -250,13 +259,80 @@ def config_record(cfg, typed, L, layers_full, **more):
     return rec
 
 
-def serving_workload(args, base, Engine):
+def expected_experts(batch, E):
+    """How many of E experts b tokens touch when every token picks one uniformly."""
+    return E * (1.0 - (1.0 - 1.0 / E) ** batch)
+
+
+def timed_decode(eng, sampler, typed, batch, context, steps, warmup, n_runs, V, rng, kernel_times=False):
+    """Decode steps of ``batch`` requests whose cache holds ``context`` positions each (pages
+    taken as a prompt's portions would take them and filled with random values), the sampled
+    tokens fed back: seconds of each of ``n_runs`` runs of ``steps`` steps, the experts touched
+    a layer (traced steps after the timed ones), and per-kernel shares if asked for."""
+    import torch
+    from spite_amd.engine.engine import StepEntry
+    from spite_amd.sampling.sampler import SamplingParams
+    slots = [eng.admit() for _ in range(batch)]
+    for s in slots:                       # in portions, as a prompt would come: pages roll off behind the chunk
+        for at in range(0, context, 2048):
+            n = min(2048, context - at)
+            eng.cache.reserve(s, n)
+            eng.cache.commit(s, n)
+    for g in eng.cache.groups:
+        g.kv.normal_(0.0, 1.0)
+    toks = rng.randint(0, V, size=batch).tolist()
+    params = [SamplingParams() for _ in range(batch)]
+    ctxs = [[] for _ in range(batch)]
+    states = [0] * batch
+
+    def one(trace=None):
+        nonlocal toks
+        logits = eng.step([StepEntry(s, [t], [0]) for s, t in zip(slots, toks)], trace=trace)
+        toks = sampler.sample(logits, params, ctxs, states)
+    for _ in range(warmup):
+        one()
+    times = []
+    for _ in range(n_runs):
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(steps):
+            one()
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t)
+    # how many experts a layer's tokens touch: traced steps (eager, the routers' choices read
+    # back once at the end) that go on from the timed ones
+    traces = []
+    for _ in range(min(steps, 16)):
+        traces.append({})
+        one(traces[-1])
+    counts = [torch.stack([torch.bincount(e.long(), minlength=typed.num_local_experts).gt(0).sum()
+                           for e in tr.get("moe_experts", [])]) for tr in traces if tr.get("moe_experts")]
+    touched = float(torch.stack(counts).float().mean()) if counts else 0.0
+    table = None
+    if kernel_times:
+        graphs, eng.use_graphs = eng.use_graphs, False
+        with KernelTimes() as kt:
+            for _ in range(4):
+                one()
+            table = kt.table(4)
+        eng.use_graphs = graphs
+    for s in slots:
+        eng.release(s)
+    return times, touched, table
+
+
+def serving_workload(args, base, Engine, reps=3):
     """``longctx`` and ``serve``: whole requests through the scheduler, the step function and the
-    sampler (``Engine.generate``), one untimed warm-up generation of a few short requests first
-    (crates/spite-bench/src/main.rs:257), then the workload once, every step timed."""
+    sampler (``Engine.generate``): one untimed warm-up generation of a few short requests first
+    (crates/spite-bench/src/main.rs:257), then the workload ``reps`` times, every step timed
+    (:285-305: the prompt steps, then the decode steps); the figures are the median repetition's
+    (:331-332).  The steps that only decode are held against the bytes they have to read
+    (``Sizes.decode_bytes_at`` of each step's requests and positions).  ``longctx`` ends with a
+    phase of its own: all requests live at the prompt's length, 64 tokens decoded together."""
     import numpy as np
     import torch
     from spite_amd.config import read_config
+    from spite_amd.sampling.sampler import Sampler
     rng = np.random.RandomState(1)
     layers_full = base["num_hidden_layers"]
     if args.workload == "longctx":
@@ -278,7 +354,9 @@ def serving_workload(args, base, Engine):
     _, typed = read_config(cfg)
     sizes = Sizes(typed, 2 if args.dtype == "bf16" else 4)
     page, budget = 64, args.prefill_tokens
-    per_req = -(-(max(lens) + new + 1) // page) * page
+    # longctx: room for the phase in which all requests decode together (warm-up, the timed runs, traced steps)
+    tail = new + 1 if args.workload != "longctx" else 2 + max(1, reps) * new + min(new, 16) + 1
+    per_req = -(-(max(lens) + tail) // page) * page
     log(f"{args.workload}: building {L} layers, {n_req} requests of {min(lens)} to {max(lens)} prompt tokens")
     t0 = time.time()
     eng = Engine(cfg, dtype=args.dtype, page_size=page, cache_tokens=n_req * per_req, max_requests=n_req,
@@ -290,13 +368,18 @@ def serving_workload(args, base, Engine):
     warm = [rng.randint(0, V, size=min(budget + 3, 300)).tolist() for _ in range(min(n_req, 4))]
     eng.generate(warm, max_tokens=4, eos_token_ids=[])
     prompts = [rng.randint(0, V, size=n).tolist() for n in lens]
-    stats, timeline = {}, []
-    torch.cuda.synchronize()
-    t = time.perf_counter()
-    outs = eng.generate(prompts, max_tokens=new, eos_token_ids=[], stats=stats, timeline=timeline)
-    torch.cuda.synchronize()
-    total = time.perf_counter() - t
-    assert all(len(o) == new for o in outs)
+    repetitions = []
+    for _ in range(max(1, reps)):
+        stats, timeline = {}, []
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        outs = eng.generate(prompts, max_tokens=new, eos_token_ids=[], stats=stats, timeline=timeline)
+        torch.cuda.synchronize()
+        repetitions.append((time.perf_counter() - t, stats, timeline))
+        assert all(len(o) == new for o in outs)
+        log(f"{args.workload}: repetition {len(repetitions)}: {repetitions[-1][0]:.2f} s")
+    seconds = [r[0] for r in repetitions]
+    total, stats, timeline = sorted(repetitions, key=lambda r: r[0])[len(repetitions) // 2]
     kinds = {"prefill": [], "decode": [], "mixed": []}
     for r in timeline:
         kind = "mixed" if r["prompt_tokens"] and r["decoded_tokens"] else "prefill" if r["prompt_tokens"] else "decode"
@@ -313,6 +396,27 @@ def serving_workload(args, base, Engine):
         for at in range(0, n, budget):
             flops += sizes.prefill_flops(min(budget, n - at), at, logit_rows=0)
     t_prompt = sum(r["wall_s"] for r in kinds["prefill"]) + sum(r["wall_s"] for r in kinds["mixed"])
+    # the steps that only decode against the bytes they have to read: every weight they use once
+    # (the experts that their tokens are expected to touch) and the cache of their requests
+    E = typed.num_local_experts
+    dec_bytes = sum(sizes.decode_bytes_at(r["starts"], expected_experts(len(r["starts"]), E)) for r in kinds["decode"])
+    dec_time = sum(r["wall_s"] for r in kinds["decode"])
+    decode_roof = {"bound": "hbm", "achieved": round(dec_bytes / max(dec_time, 1e-9) / 1e9, 1), "peak": HBM_PEAK / 1e9,
+                   "unit": "GB/s", "frac": round(dec_bytes / max(dec_time, 1e-9) / HBM_PEAK, 4),
+                   "steps": len(kinds["decode"])} if kinds["decode"] else None
+    together = None
+    if args.workload == "longctx":
+        # every request live at the prompt's length, decoding together
+        sampler = Sampler(eng.device)
+        ctx_len = max(lens)
+        t_d, touched_d, _ = timed_decode(eng, sampler, typed, n_req, ctx_len, new, 2, max(1, reps), V, rng)
+        d_med = statistics.median(t_d)
+        nb = sizes.decode_bytes(n_req, ctx_len + 2 + new // 2, touched_d)
+        together = {"batch": n_req, "context": ctx_len, "steps": new, "tok_s": round(n_req * new / d_med, 1),
+                    "ms_per_step": round(d_med / new * 1e3, 3), "frac_of_hbm_peak": round(nb / (d_med / new) / HBM_PEAK, 4),
+                    "runs_ms": [round(x / new * 1e3, 3) for x in t_d]}
+        log(f"longctx: {n_req} requests decoding together at {ctx_len}: {together['ms_per_step']} ms a step, "
+            f"{together['tok_s']} tok/s, {together['frac_of_hbm_peak']} of the HBM peak")
     out = {
         "metric": f"{args.workload}: tokens a second of whole requests through the scheduler "
                   f"({n_req} requests, prompts of {min(lens)} to {max(lens)} tokens, {new} new tokens each)",
@@ -322,7 +426,8 @@ def serving_workload(args, base, Engine):
         "data": "synthetic: random weights N(0,0.02), uniform-random token ids",
         "config": config_record(cfg, typed, L, layers_full, model=model, global_batch=n_req, seq_len=max(lens) + new,
                                 max_batch_tokens=budget),
-        "seconds": round(total, 3),
+        "seconds": round(total, 3), "runs_s": [round(x, 3) for x in seconds],
+        "decode_roofline": decode_roof, "decode_together": together,
         "prefill_tps": round(prefill_tps, 1) if prefill_tps else None,
         "decode_tps": round(decode_tps, 1) if decode_tps else None,
         "prompt_frac_of_mfma_peak": round(flops / max(t_prompt, 1e-9) / MFMA_PEAK[args.dtype], 4),
@@ -334,10 +439,11 @@ def serving_workload(args, base, Engine):
         "preemptions": stats["preemptions"],
         "peak_memory_gib": round(torch.cuda.max_memory_allocated() / 2**30, 1),
     }
-    log(f"{args.workload}: {total:.2f} s; prefill {out['prefill_tps']} tok/s, decode {out['decode_tps']} tok/s, "
-        f"ttft {out['ttft_ms']}, steps {out['step_ms']}, host {out['host_ms_per_step']}")
-    print(json.dumps(out))
-    return 0
+    log(f"{args.workload}: {total:.2f} s (runs {out['runs_s']}); prefill {out['prefill_tps']} tok/s, decode {out['decode_tps']} tok/s "
+        f"({decode_roof['frac'] if decode_roof else None} of the HBM peak), ttft {out['ttft_ms']}, steps {out['step_ms']}, "
+        f"host {out['host_ms_per_step']}")
+    del eng
+    return out
 
 
 def main() -> int:
@@ -365,6 +471,8 @@ def main() -> int:
     ap.add_argument("--new-tokens", type=int, default=None, help="longctx / serve: tokens generated per request")
     ap.add_argument("--no-graphs", action="store_true", help="run decode steps eagerly (for kernel traces)")
     ap.add_argument("--no-peaks", action="store_true", help="skip the measurement of the memory's and the product's rates")
+    ap.add_argument("--no-workloads", action="store_true",
+                    help="the default run alone, without the longctx and serve workloads behind it")
     ap.add_argument("--kernel-times", action="store_true",
                     help="after the timed runs: eager steps with an event pair around every kernel call, shares per kernel")
     ap.add_argument("--phase", default="all", choices=["all", "decode", "prefill", "sampling"],
@@ -384,7 +492,8 @@ def main() -> int:
     if args.phase == "sampling":
         return sampling_only(base["vocab_size"], args.batch, args.steps)
     if args.workload != "decode":
-        return serving_workload(args, base, Engine)
+        print(json.dumps(serving_workload(args, base, Engine, args.runs)))
+        return 0
     layers_full = base["num_hidden_layers"]
     L = args.layers or layers_full
     cfg = dict(base, num_hidden_layers=L, no_rope_layers=None)
@@ -466,57 +575,8 @@ def main() -> int:
         return 0
 
     # ---- decode at a fixed batch
-    def fill_context(slots):
-        for s in slots:                       # in portions, as a prompt would come: pages roll off behind the chunk
-            for at in range(0, args.context, 2048):
-                n = min(2048, args.context - at)
-                eng.cache.reserve(s, n)
-                eng.cache.commit(s, n)
-        for g in eng.cache.groups:
-            g.kv.normal_(0.0, 1.0)
-
     def decode(batch, steps, warmup, n_runs, kernel_times=False):
-        slots = [eng.admit() for _ in range(batch)]
-        fill_context(slots)
-        toks = rng.randint(0, V, size=batch).tolist()
-        params = [SamplingParams() for _ in range(batch)]
-        ctxs = [[] for _ in range(batch)]
-        states = [0] * batch
-
-        def one(trace=None):
-            nonlocal toks
-            logits = eng.step([StepEntry(s, [t], [0]) for s, t in zip(slots, toks)], trace=trace)
-            toks = sampler.sample(logits, params, ctxs, states)
-        for _ in range(warmup):
-            one()
-        times = []
-        for _ in range(n_runs):
-            torch.cuda.synchronize()
-            t = time.perf_counter()
-            for _ in range(steps):
-                one()
-            torch.cuda.synchronize()
-            times.append(time.perf_counter() - t)
-        # how many experts a layer's tokens touch: traced steps (eager, the routers' choices read
-        # back once at the end) that go on from the timed ones
-        traces = []
-        for _ in range(min(steps, 16)):
-            traces.append({})
-            one(traces[-1])
-        counts = [torch.stack([torch.bincount(e.long(), minlength=typed.num_local_experts).gt(0).sum()
-                               for e in tr.get("moe_experts", [])]) for tr in traces if tr.get("moe_experts")]
-        touched = float(torch.stack(counts).float().mean()) if counts else 0.0
-        table = None
-        if kernel_times:
-            graphs, eng.use_graphs = eng.use_graphs, False
-            with KernelTimes() as kt:
-                for _ in range(4):
-                    one()
-                table = kt.table(4)
-            eng.use_graphs = graphs
-        for s in slots:
-            eng.release(s)
-        return times, touched, table
+        return timed_decode(eng, sampler, typed, batch, args.context, steps, warmup, n_runs, V, rng, kernel_times)
 
     times, touched, table = decode(args.batch, args.steps, args.warmup, runs, args.kernel_times)
     dt = statistics.median(times)
@@ -564,6 +624,30 @@ def main() -> int:
     }
     if table:
         out["decode_kernels"] = table
+    if args.phase == "all" and not args.no_workloads:
+        # the other two workloads, on engines of their own once this one's memory is free: whole
+        # requests through the scheduler; a failure leaves null and its reason on stderr
+        import copy
+        import gc
+        del eng, sampler
+        gc.collect()
+        torch.cuda.empty_cache()
+        out["workloads"] = {}
+        for name in ("longctx", "serve"):
+            w_args = copy.copy(args)
+            w_args.workload, w_args.layers, w_args.experts, w_args.moe_step = name, None, None, None
+            try:
+                full = serving_workload(w_args, base, Engine, args.runs)
+                keep = ("value", "unit", "seconds", "runs_s", "prefill_tps", "decode_tps", "decode_roofline", "decode_together",
+                        "prompt_frac_of_mfma_peak", "ttft_ms", "step_ms", "peak_pages", "pool_pages", "preemptions")
+                out["workloads"][name] = dict({k: full[k] for k in keep}, layers=full["config"]["layers"],
+                                              experts=full["config"]["experts"], requests=full["config"]["global_batch"],
+                                              seq_len=full["config"]["seq_len"])
+            except Exception as e:          # noqa: BLE001 - the headline must still be printed
+                log(f"workload {name} failed: {type(e).__name__}: {e}")
+                out["workloads"][name] = None
+            gc.collect()
+            torch.cuda.empty_cache()
     print(json.dumps(out))
     return 0
 

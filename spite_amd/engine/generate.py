@@ -32,8 +32,8 @@ def generate(engine, prompts: Sequence[Sequence[int]], max_tokens: int = 16, tem
     (``ttft_s``, in the order of the prompts, from the call's start) and the most pages that
     each group of layers held (``peak_pages``).  ``timeline`` (a list) receives one record a
     step: wall seconds, GPU seconds between the step's first and last kernel, prompt tokens and
-    decoded tokens in it (the sampled tokens come back to the host every step, so a step's wall
-    time includes all of its GPU work)."""
+    decoded tokens in it and the position at which every entry began (the sampled tokens come
+    back to the host every step, so a step's wall time includes all of its GPU work)."""
     import time
     import torch
     t_begin = time.perf_counter()
@@ -90,7 +90,7 @@ def generate(engine, prompts: Sequence[Sequence[int]], max_tokens: int = 16, tem
                 timeline.append({"wall_s": now - t_step, "gpu_s": ev0.elapsed_time(ev1) * 1e-3,
                                  "prompt_tokens": sum(len(b.tokens) for b in batch if b.start < results[b.request_id].n_prompt),
                                  "decoded_tokens": sum(1 for b in batch if b.start >= results[b.request_id].n_prompt),
-                                 "entries": len(batch)})
+                                 "entries": len(batch), "starts": [b.start for b in batch]})
         for o in outs:
             res = results[o.request_id]
             if o.token >= 0:
