@@ -172,6 +172,7 @@ class Engine:
             self._source = FolderSource(model, spec.strip_prefixes, spec.ignore_prefixes)
         bind(self.model, self._source, ckpt_dtype)
         torch.cuda.empty_cache()
+        self.slow_paths = self._report_slow_paths()
         self._arenas = [Workspace(self.device, workspace_bytes), Workspace(self.device, workspace_bytes)]
         self._step_ws = Workspace(self.device, workspace_bytes)
         self._pin = None
@@ -182,6 +183,27 @@ class Engine:
         self._graphs: Dict[tuple, object] = {}     # shape of a decode step -> (segments, state), "seen" once, or "eager" for good
         self._graph_stamp = None
         self.graph_replays = 0
+
+    def _report_slow_paths(self):
+        """Says once, on standard error, which parts of this model will run a kernel far slower
+        than the one meant for them, and why (a size one step off what the MFMA kernels take costs
+        an order of magnitude, and nothing else would tell).  Returns {message: [blocks]}."""
+        found: Dict[str, list] = {}
+        if self.env.dtype != torch.bfloat16:
+            return found
+        for i, block in enumerate(self.model.blocks):
+            for what, part, _ in block.children:
+                for note in part.slow_paths(self.page_size):
+                    found.setdefault(f"{what}: {note}", []).append(i)
+        for what, part in (("embedding", self.model.embedding), ("head", self.model.head)):
+            for note in part.slow_paths(self.page_size):
+                found.setdefault(f"{what}: {note}", []).append(-1)
+        if found:
+            import sys
+            for note, blocks in found.items():
+                where = "" if blocks == [-1] else f" (blocks {blocks[0]}" + (f" to {blocks[-1]}, {len(blocks)} of them)" if len(blocks) > 1 else ")")
+                print(f"[spite_amd] slow path: {note}{where}", file=sys.stderr, flush=True)
+        return found
 
     # ------------------------------------------------------------------ weights
     def tensor_names(self):

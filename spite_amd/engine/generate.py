@@ -74,7 +74,7 @@ def generate(engine, prompts: Sequence[Sequence[int]], max_tokens: int = 16, tem
             logits = engine.step(entries, commit=False)
             wanted = [b.request_id for b in batch if b.wants_logits]
             states = [rng[r] for r in wanted]
-            toks = sampler.sample(logits, [params[r] for r in wanted], [context[r] for r in wanted], states)
+            toks = sampler.sample(logits, [params[r] for r in wanted], [context[r] for r in wanted], states, keys=wanted)
             for r, s in zip(wanted, states):
                 rng[r] = s
             if timeline is not None:
@@ -98,6 +98,7 @@ def generate(engine, prompts: Sequence[Sequence[int]], max_tokens: int = 16, tem
                 context[o.request_id].append(o.token)
             if o.done:
                 res.finish_reason = o.finish_reason
+                sampler.forget(o.request_id)
     if stats is not None:
         stats.update(steps=n_steps, tokens=n_tokens, preemptions=sched.n_preemptions,
                      ttft_s=[first_token.get(r) for r in order], peak_pages=peak,

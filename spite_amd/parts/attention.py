@@ -92,6 +92,21 @@ class Attention(Mixer):
             self.w_qnorm, self.w_knorm = t["q_norm"].contiguous(), t["k_norm"].contiguous()
         self.position.load({k[len("position."):]: v for k, v in t.items() if k.startswith("position.")})
 
+    def slow_paths(self, page_size):
+        notes = []
+        if self.env.dtype == torch.bfloat16:
+            why = []
+            if self.hd not in (64, 128):
+                why.append(f"head size {self.hd} (the MFMA kernels have 64 and 128)")
+            if page_size % 32:
+                why.append(f"pages of {page_size} keys (they take multiples of 32)")
+            if why:
+                notes.append("attention runs on plain FMAs: " + ", ".join(why))
+            for name, w in (("q/k/v projection", self.wqkv), ("output projection", self.wo)):
+                if w is not None:
+                    notes += w.slow_reason(name)
+        return notes
+
     def cache_need(self):
         return CacheNeed(kv=KVNeed(self.G, self.hd, self.visibility, self.span))
 

@@ -106,6 +106,12 @@ class Part:
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         """``tensors``: local name -> tensor on the GPU, already in its resident dtype."""
 
+    def slow_paths(self, page_size: int) -> List[str]:
+        """After loading: one line for every way in which this part, at its sizes and the cache's
+        page size, will run a kernel far slower than the one meant for it (a product or an
+        attention on plain FMAs in a bfloat16 run).  The engine prints them once when it is built."""
+        return []
+
 
 class Norm(Part):
     def can_project(self, proj) -> bool:

@@ -51,5 +51,8 @@ class LinearHead(Head):
         if self.tied:
             self.weight = embedding.table
 
+    def slow_paths(self, page_size):
+        return self.weight.slow_reason("output matrix") if isinstance(self.weight, Weight) else []
+
     def forward(self, x, logits, ctx):
         linear(x, self.weight, logits, ws=ctx.ws)

@@ -40,6 +40,9 @@ class DenseGLU(FeedForward):
         self.w_gate_up = Weight(torch.cat([t["gate_proj"].to(dt), t["up_proj"].to(dt)], dim=0), self.F % 16 == 0)
         self.w_down = Weight(t["down_proj"])
 
+    def slow_paths(self, page_size):
+        return self.w_gate_up.slow_reason("gate/up projection") + self.w_down.slow_reason("down projection")
+
     def forward(self, x, x32, ctx, projected=None):
         T = x.shape[0]
         act = ctx.ws.take((T, self.F), x.dtype)
@@ -85,6 +88,11 @@ class MoeTop1Sigmoid(FeedForward):
             self.fused_shared = False
             self.w_gate_up, self.w_down = Weight(gu, self.F % 16 == 0), Weight(dn)
             self.ws_gate_up, self.ws_down = Weight(sgu, self.Fs % 16 == 0), Weight(sdn)
+
+    def slow_paths(self, page_size):
+        ws = [("experts' gate/up", self.w_gate_up), ("experts' down", self.w_down),
+              ("shared expert's gate/up", self.ws_gate_up), ("shared expert's down", self.ws_down)]
+        return [n for name, w in ws if w is not None for n in w.slow_reason(name)]
 
     def _few_rows_a_group(self, T: int) -> bool:
         """Whether a routed group of a step of T tokens is unlikely to hold more than 16 rows
@@ -136,15 +144,17 @@ class MoeTop1Sigmoid(FeedForward):
             linear(act, self.w_down, y, offsets=offsets, n_groups=E, y_rows=dst, rows=T, max_rows=16, ws=ws)
             linear(act[T:], self.w_down.group(E), y, y_rows=dst[T:], rows=T, ws=ws)
             return (y[:T], y[T:])
-        shape = grouped_tile_shape(T, E, groups - E) if T > SKINNY_MAX_ROWS else 0
+        # the tile of either product, by the rounds that its tiles make on the chip (gate and up
+        # rows share a tile of 512 W rows: 256 columns of the result; the down product's tile has 512)
+        shape = grouped_tile_shape(T, E, groups - E, col_tiles=-(-F // 256)) if T > SKINNY_MAX_ROWS else 0
+        shape_down = grouped_tile_shape(T, E, groups - E, col_tiles=-(-d // 512)) if T > SKINNY_MAX_ROWS else 0
         # every token goes to one expert: at most min(T, E) of their groups hold rows, and the shared one
         live = min(T, E) + (groups - E)
         linear(x, self.w_gate_up, act, glu=True, offsets=offsets, n_groups=groups, a_rows=src, a_scale=scale, rows=n,
                max_rows=T, tile_shape=shape, live_groups=live, ws=ws)
         # slot s writes row dst[s]: rows [0,T) the routed result per token, rows [T,2T) the shared one
-        # (the down product has too few column tiles for the larger row tile to pay)
         linear(act, self.w_down, y, offsets=offsets, n_groups=groups, y_rows=dst, rows=n, max_rows=T,
-               tile_shape=shape if shape == 4 else 0, live_groups=live, ws=ws)
+               tile_shape=shape_down, live_groups=live, ws=ws)
         if self.fused_shared:
             return (y[:T], y[T:])
         act_s = ws.take((T, self.Fs), x.dtype)

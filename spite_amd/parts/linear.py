@@ -7,6 +7,7 @@
 from __future__ import annotations
 
 import math
+from typing import List
 
 import torch
 
@@ -43,6 +44,14 @@ class Weight:
                           and w.shape[-2] % 16 == 0 and w.shape[-1] % 64 == 0)
         self.data = hipops.operand_order(w) if self.tiled else w
 
+    def slow_reason(self, name: str) -> List[str]:
+        """Why products with this weight will not run on the matrix units in a bfloat16 run."""
+        if self.dtype == torch.bfloat16 and self.shape[-1] % 8:
+            return [f"{name} {self.shape}: rows of {self.shape[-1]} are no multiple of 8, its products run on plain FMAs"]
+        if self.dtype == torch.float32:
+            return [f"{name} {self.shape}: kept in 32-bit by the checkpoint, its products run on plain FMAs"]
+        return []
+
     def group(self, g: int) -> "Weight":
         """Group ``g`` of a stack of matrices ``[groups, out, in]`` as a weight of its own (the same
         memory)."""
@@ -51,7 +60,12 @@ class Weight:
         return one
 
 
-def grouped_tile_shape(tokens: int, groups: int, whole_groups: int = 0) -> int:
+# what a tile of 160 rows costs against one of 128 (a tile's time is a fixed part and a part per
+# 16 rows, 38 and 8.5 us at K = 5,120 on an MI355X: (38 + 85) / (38 + 68))
+TILE_160_COST = 1.16
+
+
+def grouped_tile_shape(tokens: int, groups: int, whole_groups: int = 0, col_tiles: int = 0, cus: int = 0) -> int:
     """Which tile of the prefill product suits ``tokens`` rows that spread evenly over ``groups``
     groups (experts that a router picks), beside ``whole_groups`` groups that take every row.
     A group costs whole row tiles, each of which streams the group's weights once.
@@ -62,9 +76,13 @@ def grouped_tile_shape(tokens: int, groups: int, whole_groups: int = 0) -> int:
       every row do not need many of those small tiles.  (With 128 experts there are workgroups
       enough: measured no gain.)
     * Else 128 rows a tile (shape 1), or 160 (shape 3, about a sixth dearer per tile) where that
-      saves tiles: with groups of about 128 rows half of them need a second tile of 128, almost
-      none a second one of 160.  The expected number of tiles of each shape decides, group sizes
-      taken as normal around tokens/groups."""
+      saves time: with groups of about 128 rows half of them need a second tile of 128, almost
+      none a second one of 160.  The expected number of row tiles of each shape, group sizes
+      taken as normal around tokens/groups, times ``col_tiles`` column tiles, runs on ``cus``
+      compute units in whole rounds (a workgroup a unit): the fewer rounds, each at its tile's
+      cost, win.  (Measured at widths of 4,096 to 6,144, 8 and 16 experts of 8,192 and 14,336:
+      the choice by rounds was the faster tile in all eight products.)  Without ``col_tiles`` the
+      row tiles alone are compared."""
     if groups <= 0 or tokens <= 0:
         return 1
     mean = tokens / groups
@@ -78,6 +96,10 @@ def grouped_tile_shape(tokens: int, groups: int, whole_groups: int = 0) -> int:
             extra += 0.5 * math.erfc((k * rows_per_tile + 0.5 - mean) / (sd * math.sqrt(2.0)))
             k += 1
         return groups * (1.0 + extra) + whole_groups * -(-tokens // rows_per_tile)
+    if col_tiles > 0:
+        cus = cus or hipops.cu_count()
+        rounds = lambda rows_per_tile: math.ceil(tiles(rows_per_tile) * col_tiles / cus - 1e-9)
+        return 3 if TILE_160_COST * rounds(160) < rounds(128) else 1
     return 3 if 1.17 * tiles(160) < tiles(128) else 1
 
 

@@ -19,6 +19,14 @@ def test_tile_shape_follows_the_expected_number_of_row_tiles():
     assert grouped_tile_shape(0, 16, 1) == 1 and grouped_tile_shape(100, 0) == 1
 
 
+def test_tile_shape_by_the_rounds_its_tiles_make():
+    # the eight products measured at 2,048 tokens on 256 compute units: (experts, column tiles) -> the faster tile
+    for E, cols, want in ((16, 32, 3), (16, 10, 1), (8, 32, 3), (8, 8, 3), (8, 12, 1), (8, 56, 1)):
+        assert grouped_tile_shape(2048, E, 1, col_tiles=cols, cus=256) == want, (E, cols)
+    # a short prompt still takes the small tile, whatever the columns
+    assert grouped_tile_shape(256, 16, 1, col_tiles=10, cus=256) == 4
+
+
 def test_runs_of_a_split_product_are_never_empty():
     from spite_amd.csrc.hipops import tiled_k_runs
     for M in (65, 100, 256, 700, 2048):
