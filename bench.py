@@ -279,7 +279,8 @@ def timed_decode(eng, sampler, typed, batch, context, steps, warmup, n_runs, V, 
             eng.cache.reserve(s, n)
             eng.cache.commit(s, n)
     for g in eng.cache.groups:
-        g.kv.normal_(0.0, 1.0)
+        for half in g.halves():
+            half.normal_(0.0, 1.0)
     toks = rng.randint(0, V, size=batch).tolist()
     params = [SamplingParams() for _ in range(batch)]
     ctxs = [[] for _ in range(batch)]
@@ -547,7 +548,8 @@ def main() -> int:
     if args.phase != "decode":
         if args.prefill_context:
             for g in eng.cache.groups:
-                g.kv.normal_(0.0, 1.0)
+                for half in g.halves():
+                    half.normal_(0.0, 1.0)
         prefill_once()
         pre_runs = [prefill_once() for _ in range(runs)]
         pre = statistics.median(pre_runs)

@@ -2,10 +2,11 @@
 the host-side bookkeeping in the native cache manager.
 
 Layers are grouped by what they need: the same number of kv heads, head size and
-visibility (every key, the query's chunk, a window).  A group's pool is one tensor
-``[layers, 2, pages, kv_heads, page_size, head_dim]`` (the value half is used transposed,
-``[pages, kv_heads, head_dim, page_size]``); a page is the same row range in every layer of
-the group, so one block table serves all of them.
+visibility (every key, the query's chunk, a window).  A group's pool is two tensors, keys
+``[layers, pages, kv_heads, page_size, key width]`` and values, transposed,
+``[layers, pages, kv_heads, value width, page_size]`` (a mixer may ask for values of another
+width than its keys); a page is the same row range in every layer of the group, so one block
+table serves all of them.
 """
 from __future__ import annotations
 
@@ -32,10 +33,15 @@ class OutOfPages(CacheError):
 
 @dataclass
 class Group:
-    key: tuple                   # (kv heads, head size, visibility, span)
+    key: tuple                   # (kv heads, key width, visibility, span, value width)
     cache_ids: List[int]
     n_pages: int
-    kv: Optional[torch.Tensor]   # [layers, 2, pages, G, page_size, hd]
+    k: Optional[torch.Tensor] = None     # [layers, pages, G, page_size, key width]
+    v: Optional[torch.Tensor] = None     # [layers, pages, G, value width, page_size]: values lie transposed
+
+    def halves(self):
+        """The pool's tensors (to fill or to poison all of it)."""
+        return (self.k, self.v)
 
 
 class PagedCache:
@@ -55,7 +61,7 @@ class PagedCache:
             if need is None or need.kv is None:
                 continue
             kv = need.kv
-            key = (kv.n_kv_heads, kv.head_dim, kv.visibility, kv.span if kv.visibility != "full" else 0)
+            key = (kv.n_kv_heads, kv.head_dim, kv.visibility, kv.span if kv.visibility != "full" else 0, kv.value_dim)
             if key not in by_key:
                 by_key[key] = len(self.groups)
                 self.groups.append(Group(key, [], 0, None))
@@ -93,8 +99,9 @@ class PagedCache:
         self.states: Dict[int, torch.Tensor] = {}
         if allocate:
             for g in self.groups:
-                G, hd = g.key[0], g.key[1]
-                g.kv = torch.zeros((len(g.cache_ids), 2, g.n_pages, G, self.page_size, hd), dtype=dtype, device=device)
+                G, kd, vd = g.key[0], g.key[1], g.key[4]
+                g.k = torch.zeros((len(g.cache_ids), g.n_pages, G, self.page_size, kd), dtype=dtype, device=device)
+                g.v = torch.zeros((len(g.cache_ids), g.n_pages, G, vd, self.page_size), dtype=dtype, device=device)
             for cid, need in enumerate(needs):
                 if need is not None and need.state is not None:
                     self.states[cid] = torch.zeros((self.max_requests, *need.state.shape),
@@ -222,11 +229,10 @@ class PagedCache:
         """Whether this cache's pages are kept in the MFMA attention kernels' operand order
         (bfloat16, head size and page size multiples of 32) rather than row-major."""
         g = self.groups[self._group_of[cache_id]]
-        return hipops.kv_tiled_ok(self.dtype, g.key[1], self.page_size)
+        return g.key[1] == g.key[4] and hipops.kv_tiled_ok(self.dtype, g.key[1], self.page_size)
 
     def layer_pages(self, cache_id: int):
         g = self.groups[self._group_of[cache_id]]
         li = self._layer_in_group[cache_id]
-        G, hd = g.key[0], g.key[1]
-        # keys [pages, G, page_size, hd]; values transposed in the same bytes: [pages, G, hd, page_size]
-        return g.kv[li, 0], g.kv[li, 1].view(g.n_pages, G, hd, self.page_size)
+        # keys [pages, G, page_size, key width]; values transposed: [pages, G, value width, page_size]
+        return g.k[li], g.v[li]

@@ -30,7 +30,8 @@ void attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_p
                         const bf16* __restrict__ v_pages, float* __restrict__ part, bf16* __restrict__ out,
                         const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                         const int* __restrict__ block_table, int max_blocks, int H, int G, int ps, int vis,
-                        int span, float scale_log2e, float cap_ratio, int n_splits) {
+                        int span, float scale_log2e, float cap_ratio, int n_splits,
+                        const float* __restrict__ slopes, float inv_scale) {
     constexpr int NC = HD / 32;      // 32-wide chunks of the head for the score product
     constexpr int ND = HD / 16;      // 16-row tiles of the output
     constexpr int ROW = HD + 2;      // partial record: output, max, sum
@@ -42,6 +43,8 @@ void attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_p
     const int p = positions[t];
     const int lo = sp_first_visible(p, vis, span);
     const int* bt = block_table + (size_t)seq_of_token[t] * max_blocks;
+    // a bias slope * (key - query position) on the scaled score of head n, as an addend of the raw score
+    const float slope = (slopes && n < QH) ? slopes[g * QH + n] * inv_scale : 0.f;
 
     const int b_first = lo / 32, b_last = p / 32;
     const int nblk = b_last - b_first + 1;
@@ -105,7 +108,7 @@ void attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_p
             for (int i = 0; i < 4; ++i) {
                 const int j = key0 + qd * 8 + tt * 4 + i;
                 ok[tt][i] = j >= lo && j <= p;
-                float raw = s[tt][i];
+                float raw = s[tt][i] + slope * (float)(j - p);
                 // a cap on the scores: cap * tanh(score * scale / cap), with cap_ratio = scale / cap
                 if (cap_ratio > 0.f) raw = tanhf(raw * cap_ratio) / cap_ratio;
                 const float v = ok[tt][i] ? (page < 0 ? NAN : raw * scale_log2e) : -INFINITY;
@@ -238,7 +241,7 @@ extern "C" size_t spite_attn_decode_workspace(int T, int H, int hd, int n_splits
 extern "C" int spite_attn_decode(const void* q, const void* k_pages, const void* v_pages, void* out, void* workspace,
                                  const int* positions, const int* seq_of_token, const int* block_table,
                                  int max_blocks, int T, int H, int G, int hd, int page_size, int vis, int span,
-                                 float scale, float softcap, int n_splits, hipStream_t st) {
+                                 float scale, float softcap, const float* slopes, int n_splits, hipStream_t st) {
     SP_REQUIRE(softcap >= 0.f && scale > 0.f, "attn_decode: scale %g, score cap %g", scale, softcap);
     SP_REQUIRE(T >= 0 && H > 0 && G > 0 && H % G == 0, "attn_decode: %d query heads over %d kv heads", H, G);
     SP_REQUIRE(H / G <= 16, "attn_decode: %d query heads per kv head, at most 16", H / G);
@@ -253,13 +256,13 @@ extern "C" int spite_attn_decode(const void* q, const void* k_pages, const void*
     const size_t sh = (size_t)4 * 16 * (hd + 2) * sizeof(float);
     if (hd == 128) {
         attn_decode_kernel<128><<<grid, 256, sh, st>>>((const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages,
-            (float*)workspace, (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, cr, n_splits);
+            (float*)workspace, (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, cr, n_splits, slopes, 1.0f / scale);
         SP_LAUNCH_CHECK("attn_decode");
         if (n_splits > 1)
             attn_decode_combine_kernel<128><<<dim3(T, H), 128, 0, st>>>((const float*)workspace, (bf16*)out, H, n_splits);
     } else {
         attn_decode_kernel<64><<<grid, 256, sh, st>>>((const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages,
-            (float*)workspace, (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, cr, n_splits);
+            (float*)workspace, (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, cr, n_splits, slopes, 1.0f / scale);
         SP_LAUNCH_CHECK("attn_decode");
         if (n_splits > 1)
             attn_decode_combine_kernel<64><<<dim3(T, H), 64, 0, st>>>((const float*)workspace, (bf16*)out, H, n_splits);
@@ -305,5 +308,5 @@ extern "C" int spite_attn_decode_static(const void* q, const void* k_pages, cons
     SP_REQUIRE(e == hipSuccess && ptr != nullptr, "attn_decode_static: no address for the scratch array: %s",
                hipGetErrorString(e));
     return spite_attn_decode(q, k_pages, v_pages, out, ptr, positions, seq_of_token, block_table, max_blocks, T, H, G,
-                             hd, page_size, vis, span, scale, 0.f, n_splits, st);
+                             hd, page_size, vis, span, scale, 0.f, nullptr, n_splits, st);
 }

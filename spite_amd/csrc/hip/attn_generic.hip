@@ -5,7 +5,8 @@
 // the request's block table.  Keys are walked in tiles of 64 that start at first_visible(p),
 // so the order of every sum depends on p alone: a token gives the same bits whether it comes
 // in a whole prompt, a portion or alone.  Scores, running maximum, running sum and the
-// output are fp32; exp is the accurate one.
+// output are fp32; exp is the accurate one.  Options: a smooth cap on the scaled scores, and
+// per-head slopes of a bias slope * (key position - query position) added before the cap.
 #include "common.h"
 
 #define ATT_MAX_D 8   // head sizes up to 512
@@ -15,7 +16,8 @@ __global__ __launch_bounds__(64)
 void attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
                          T* __restrict__ out, const int* __restrict__ positions,
                          const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
-                         int max_blocks, int H, int G, int hd, int ps, int vis, int span, float scale, float softcap, int kv_tiled) {
+                         int max_blocks, int H, int G, int hd, int ps, int vis, int span, float scale, float softcap, int kv_tiled,
+                         const float* __restrict__ slopes) {
     extern __shared__ float smem[];
     float* q_sh = smem;                 // [hd]
     float* p_sh = smem + hd;            // [64]
@@ -26,6 +28,7 @@ void attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
     const int p = positions[t];
     const int* bt = block_table + (size_t)seq_of_token[t] * max_blocks;
     const int lo = sp_first_visible(p, vis, span);
+    const float slope = slopes ? slopes[h] : 0.f;      // a bias slope * (key - query position) on the scaled score
     const T* qr = q + ((size_t)t * H + h) * hd;
     for (int c = lane; c < hd; c += 64) q_sh[c] = to_f32<T>(qr[c]);
     __syncthreads();
@@ -49,7 +52,7 @@ void attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
                 const T* kr = k_pages + row;
                 float acc = 0.f;
                 for (int c = 0; c < hd; ++c) acc = fmaf(q_sh[c], to_f32<T>(kr[sp_k_index(j % ps, c, hd, kv_tiled)]), acc);
-                s = acc * scale;
+                s = acc * scale + slope * (float)(j - p);
                 if (softcap > 0.f) s = softcap * tanhf(s / softcap);       // scores capped smoothly at +-softcap
             }
         }
@@ -90,7 +93,7 @@ void attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
 extern "C" int spite_attn_generic(const void* q, const void* k_pages, const void* v_pages, void* out, int dtype,
                                   const int* positions, const int* seq_of_token, const int* block_table,
                                   int max_blocks, int T, int H, int G, int hd, int page_size, int vis, int span,
-                                  float scale, float softcap, int kv_tiled, hipStream_t st) {
+                                  float scale, float softcap, const float* slopes, int kv_tiled, hipStream_t st) {
     SP_REQUIRE(softcap >= 0.f, "attention: score cap %g", softcap);
     SP_REQUIRE(T >= 0 && H > 0 && G > 0 && H % G == 0, "attention: %d query heads over %d kv heads", H, G);
     SP_REQUIRE(hd > 0 && hd <= 64 * ATT_MAX_D, "attention: head size %d, at most %d", hd, 64 * ATT_MAX_D);
@@ -104,10 +107,10 @@ extern "C" int spite_attn_generic(const void* q, const void* k_pages, const void
     const size_t sh = (size_t)(hd + 64) * sizeof(float) + 64 * sizeof(long long) + 64 * sizeof(int) + 8;
     if (dtype == SP_F32)
         attn_generic_kernel<float><<<grid, 64, sh, st>>>((const float*)q, (const float*)k_pages, (const float*)v_pages,
-            (float*)out, positions, seq_of_token, block_table, max_blocks, H, G, hd, page_size, vis, span, scale, softcap, kv_tiled);
+            (float*)out, positions, seq_of_token, block_table, max_blocks, H, G, hd, page_size, vis, span, scale, softcap, kv_tiled, slopes);
     else if (dtype == SP_BF16)
         attn_generic_kernel<bf16><<<grid, 64, sh, st>>>((const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages,
-            (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, hd, page_size, vis, span, scale, softcap, kv_tiled);
+            (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, hd, page_size, vis, span, scale, softcap, kv_tiled, slopes);
     else return sp_fail("attention: unknown dtype %d", dtype);
     SP_LAUNCH_CHECK("attn_generic");
     return 0;

@@ -41,11 +41,11 @@ def lib():
             "spite_convert": [P, I, P, I, c_size_t, P],
             "spite_randn_fill": [P, I, c_size_t, ctypes.c_ulonglong, ctypes.c_ulonglong, F, F, P],
             "spite_gemm_generic": [P, I, P, L, I, P, I, I, I, I, I, P, I, P, P, P, I, P],
-            "spite_attn_generic": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, F, I, P],
+            "spite_attn_generic": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, F, P, I, P],
             "spite_sample_rows": [P, I, I, I, P, P, P, P],
             "spite_filter_rows": [P, I, I, I, P, P, P, P],
             "spite_gemm_skinny": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, I, I, I, P],
-            "spite_attn_decode": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, F, I, P],
+            "spite_attn_decode": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, F, P, I, P],
             "spite_gemm_mfma": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, P],
             "spite_gemm_tiled": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, P],
             "spite_gemm_tiled_split": [P, I, P, P, I, I, I, I, I, I, P, P],
@@ -268,11 +268,12 @@ def gemm_generic(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_s
 
 
 def attn_generic(q, k_pages, v_pages, out, positions, seq_of_token, block_table, T, H, G, hd, page_size,
-                 vis, span, scale, kv_tiled=False, softcap=0.0):
+                 vis, span, scale, kv_tiled=False, softcap=0.0, slopes=None):
     """Attention over the paged cache, any mix of portions and single tokens.  q/out
     [T,H*hd]; block_table int32 [n_seqs, max_blocks].  ``kv_tiled``: the pages are in operand
-    order (``kv_operand_order``).  ``softcap`` > 0 (here and in the MFMA kernels): the scaled scores
-    are capped smoothly, ``softcap * tanh(score / softcap)``, before the softmax."""
+    order (``kv_operand_order``).  Here and in the MFMA kernels: ``slopes`` (fp32 [H]) adds
+    slopes[head] * (key position - query position) to the scaled scores; ``softcap`` > 0 then caps
+    them smoothly, ``softcap * tanh(score / softcap)``, before the softmax."""
     if q.numel() < T * H * hd or out.numel() < T * H * hd:
         raise KernelError("attention: q or out too small")
     _check_pages(k_pages, v_pages, G, page_size, hd, "attention")
@@ -283,7 +284,7 @@ def attn_generic(q, k_pages, v_pages, out, positions, seq_of_token, block_table,
         _ptr(q, "q"), _ptr(k_pages, "k_pages", dt), _ptr(v_pages, "v_pages", dt), _ptr(out, "out", dt),
         dtype_code(dt), _ptr(positions, "positions", torch.int32), _ptr(seq_of_token, "seq_of_token", torch.int32),
         _ptr(block_table, "block_table", torch.int32), block_table.shape[1], T, H, G, hd, page_size,
-        VIS[vis], int(span or 0), float(scale), float(softcap), int(bool(kv_tiled)), _stream()), "attention")
+        VIS[vis], int(span or 0), float(scale), float(softcap), _slopes(slopes, H), int(bool(kv_tiled)), _stream()), "attention")
 
 
 def sample_rows(logits, temperature, uniform, out, n_rows=None):
@@ -381,7 +382,7 @@ def attn_decode_workspace(T, H, hd, n_splits) -> int:
 
 
 def attn_decode(q, k_pages, v_pages, out, workspace, positions, seq_of_token, block_table, T, H, G, hd,
-                page_size, vis, span, scale, n_splits, softcap=0.0):
+                page_size, vis, span, scale, n_splits, softcap=0.0, slopes=None):
     """Split-KV decode attention on MFMA (bf16; head sizes 64 and 128; pages of a multiple of 32
     keys, in operand order): every row of q is one query against its request's cache."""
     if q.dtype != torch.bfloat16:
@@ -399,7 +400,7 @@ def attn_decode(q, k_pages, v_pages, out, workspace, positions, seq_of_token, bl
         _ptr(workspace, "workspace"), _ptr(positions, "positions", torch.int32),
         _ptr(seq_of_token, "seq_of_token", torch.int32), _ptr(block_table, "block_table", torch.int32),
         block_table.shape[1], T, H, G, hd, page_size, VIS[vis], int(span or 0), float(scale), float(softcap),
-        int(n_splits), _stream()), "attn_decode")
+        _slopes(slopes, H), int(n_splits), _stream()), "attn_decode")
 
 
 def gemm_mfma(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None, glu=False,

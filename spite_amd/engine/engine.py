@@ -110,14 +110,19 @@ class StepMeta:
             derived={name: (dv[f"derived:{name}"], info) for name, (_, info) in derived.items()})
         self.host_tokens = tok[:T].copy()
 
-    def layer_cache(self, cache: PagedCache, call: LayerCall) -> LayerCache:
-        state = cache.states.get(call.cache)
-        if call.cache not in cache._group_of:
-            return LayerCache(None, None, None, None, cache.page_size, call.write, state)
-        g = cache.group_of(call.cache)
-        k, v = cache.layer_pages(call.cache)
-        return LayerCache(k, v, self.slot_maps[g], self.tables[g], cache.page_size, call.write, state,
-                          cache.kv_tiled(call.cache))
+    def layer_cache(self, cache: PagedCache, call: LayerCall):
+        """The cache as the call's block sees it: one ``LayerCache``, or, for a block with several
+        caches, a dict of them by the block's names."""
+        def one(cid):
+            state = cache.states.get(cid)
+            if cid not in cache._group_of:
+                return LayerCache(None, None, None, None, cache.page_size, call.write, state)
+            g = cache.group_of(cid)
+            k, v = cache.layer_pages(cid)
+            return LayerCache(k, v, self.slot_maps[g], self.tables[g], cache.page_size, call.write, state,
+                              cache.kv_tiled(cid))
+        ids = call.cache_ids()
+        return one(ids[""]) if set(ids) == {""} else {name: one(cid) for name, cid in ids.items()}
 
 
 class Engine:

@@ -29,15 +29,20 @@ class Model:
         for i, call in enumerate(spec.order):
             if not 0 <= call.block < len(self.blocks):
                 raise ValueError(f"layer call {i} names block {call.block} of {len(self.blocks)}")
+            wanted, given = set(self.blocks[call.block].cache_needs()), set(call.cache_ids())
+            if wanted != given and not (len(wanted) == 1 and given == {""}):
+                raise ValueError(f"layer call {i}: block {call.block} has the caches {sorted(wanted)}, the call names {sorted(given)}")
         writers = {}
         for i, call in enumerate(spec.order):
             if call.write:
-                if call.cache in writers:
-                    raise ValueError(f"cache {call.cache} is written by layer calls {writers[call.cache]} and {i}")
-                writers[call.cache] = i
+                for cid in call.cache_ids().values():
+                    if cid in writers:
+                        raise ValueError(f"cache {cid} is written by layer calls {writers[cid]} and {i}")
+                    writers[cid] = i
         for i, call in enumerate(spec.order):
-            if not call.write and (call.cache not in writers or writers[call.cache] > i):
-                raise ValueError(f"layer call {i} reads cache {call.cache} before any call has written it")
+            for cid in call.cache_ids().values():
+                if not call.write and (cid not in writers or writers[cid] > i):
+                    raise ValueError(f"layer call {i} reads cache {cid} before any call has written it")
         self._writers = writers
         self._units = self._build_units()
         self.graph_safe = all(u[1] for u in self._units)
@@ -69,10 +74,15 @@ class Model:
         self.head.tie(self.embedding)
 
     def cache_needs(self) -> List[Optional[CacheNeed]]:
-        n = max((c.cache for c in self.spec.order), default=-1) + 1
+        """What every cache id asks for: what the block of the call that writes it says."""
+        n = max((cid for c in self.spec.order for cid in c.cache_ids().values()), default=-1) + 1
         needs: List[Optional[CacheNeed]] = [None] * n
         for cid, i in self._writers.items():
-            needs[cid] = self.blocks[self.spec.order[i].block].mixer.cache_need()
+            call = self.spec.order[i]
+            of_block = self.blocks[call.block].cache_needs()
+            for name, c in call.cache_ids().items():
+                if c == cid:
+                    needs[cid] = of_block[name] if name in of_block else next(iter(of_block.values()))
         return needs
 
     # ------------------------------------------------------------------ one step

@@ -69,7 +69,7 @@ class Attention(Mixer):
         self.scale = float(softmax_scale) if softmax_scale is not None else 1.0 / math.sqrt(self.hd)
         self.position = build_part("position", position, env)
         self.graph_safe = self.position.graph_safe
-        self.wqkv = self.wo = None
+        self.wqkv = self.wo = self.slopes = None
 
     def params(self):
         d, H, G, hd = self.d, self.H, self.G, self.hd
@@ -91,6 +91,9 @@ class Attention(Mixer):
         if self.qk_norm_weighted:
             self.w_qnorm, self.w_knorm = t["q_norm"].contiguous(), t["k_norm"].contiguous()
         self.position.load({k[len("position."):]: v for k, v in t.items() if k.startswith("position.")})
+        self.slopes = self.position.score_slopes(self.H)
+        if self.slopes is not None and (self.slopes.dtype != torch.float32 or self.slopes.numel() != self.H):
+            raise ValueError(f"attention: the position encoding's score slopes must be {self.H} fp32 values")
 
     def slow_paths(self, page_size):
         notes = []
@@ -125,7 +128,7 @@ class Attention(Mixer):
         scratch = ctx.ws.take((hipops.attn_decode_workspace(T, H, hd, n_splits) // 4,), torch.float32)
         hipops.attn_decode(q, cache.k_pages, cache.v_pages, o, scratch, ctx.positions, ctx.seq_of_token,
                            cache.block_table, T, H, G, hd, cache.page_size, self.visibility, self.span,
-                           self.scale, n_splits, softcap=self.score_cap)
+                           self.scale, n_splits, softcap=self.score_cap, slopes=self.slopes)
 
     def _prefill(self, q, o, ctx, cache, lead, cu_seqlens):
         """The tiled kernel over the step's entries from ``lead`` on (portions of prompts)."""
@@ -142,7 +145,7 @@ class Attention(Mixer):
             scratch = ctx.ws.take((hipops.attn_prefill_workspace(counts, H, G, hd, n_splits) // 4,), torch.float32)
         hipops.attn_prefill(q, cache.k_pages, cache.v_pages, o, ctx.positions[lead:], cu_seqlens, counts,
                             cache.block_table[lead:], H, G, hd, cache.page_size, self.visibility, self.span, self.scale,
-                            n_splits=n_splits, scratch=scratch, softcap=self.score_cap)
+                            n_splits=n_splits, scratch=scratch, softcap=self.score_cap, slopes=self.slopes)
 
     def forward(self, x, ctx, cache):
         T = x.shape[0]
@@ -178,7 +181,7 @@ class Attention(Mixer):
         else:
             hipops.attn_generic(q, cache.k_pages, cache.v_pages, o, ctx.positions, ctx.seq_of_token,
                                 cache.block_table, T, H, G, hd, cache.page_size, self.visibility, self.span,
-                                self.scale, kv_tiled=cache.tiled, softcap=self.score_cap)
+                                self.scale, kv_tiled=cache.tiled, softcap=self.score_cap, slopes=self.slopes)
         out = ws.take((T, self.d), torch.float32)
         linear(o, self.wo, out, ws=ws)
         return out

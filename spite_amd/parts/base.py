@@ -27,11 +27,17 @@ class ParamSpec:
 
 @dataclass(frozen=True)
 class KVNeed:
-    """Keys and values in pages: heads, head size and which keys a query may read."""
+    """Keys and values in pages: heads, the width of a key and of a value, and which keys a
+    query may read."""
     n_kv_heads: int
-    head_dim: int
+    head_dim: int                     # width of a key (and of a value, unless v_head_dim says otherwise)
     visibility: str = "full"          # "full" | "chunk" | "window"
     span: int = 0                     # chunk size or window
+    v_head_dim: Optional[int] = None  # width of a value where it differs from a key's (the pool's two halves are sized apart)
+
+    @property
+    def value_dim(self) -> int:
+        return self.head_dim if self.v_head_dim is None else int(self.v_head_dim)
 
 
 @dataclass(frozen=True)
@@ -58,7 +64,7 @@ class PartSpec:
 class BlockSpec:
     kind: str                    # arrangement, e.g. "prenorm"
     norm1: PartSpec
-    mixer: PartSpec
+    mixer: Any                   # a PartSpec; an arrangement with several mixers takes what it likes here (a dict of them)
     norm2: PartSpec
     ffn: PartSpec
 
@@ -66,8 +72,12 @@ class BlockSpec:
 @dataclass(frozen=True)
 class LayerCall:
     block: int                   # index into ModelSpec.blocks
-    cache: int                   # cache id; the call with write=True fills it
-    write: bool = True
+    cache: Any                   # cache id; the call with write=True fills it.  A block with several caches
+    write: bool = True           # (``Block.cache_needs``) names them all: {the block's name of a cache: cache id}
+
+    def cache_ids(self) -> Dict[str, int]:
+        """{the block's name of a cache: cache id}; a call with one id serves a block with one cache."""
+        return dict(self.cache) if isinstance(self.cache, dict) else {"": int(self.cache)}
 
 
 @dataclass
@@ -133,6 +143,12 @@ class PositionEncoding(Part):
     def kernel_args(self) -> Dict[str, Any]:
         return {"use_rope": False, "inv_freq": None, "adjacent": False}
 
+    def score_slopes(self, n_heads: int):
+        """For encodings that work on the scores instead of on q and k: an fp32 tensor [n_heads]
+        on the GPU, head h's score of (query at p, key at j) gets slopes[h] * (j - p) added (before
+        a cap, if there is one), or None.  The attention kernels take it as an option."""
+        return None
+
     def transform(self, qkv, positions, n_heads, n_kv_heads, head_dim) -> None:
         """For encodings the fused kernel does not know: change q and k of the fused
         projection's rows in place before they are normed and cached."""
@@ -183,6 +199,14 @@ class Head(Part):
 
 
 class Block(Part):
+    def cache_needs(self) -> Dict[str, CacheNeed]:
+        """What the block's parts ask of the cache manager, by names of the block's own choosing.
+        A block with one mixer has one entry (any name); a block with several mixers, or a mixer
+        with caches of two shapes, names each, and its layer calls give every name a cache id
+        (``LayerCall(block, {"attn": 0, "state": 1})``); ``forward`` then gets a dict of
+        ``LayerCache`` by those names instead of one.  Default: the ``mixer`` attribute's need."""
+        return {"": self.mixer.cache_need()}
+
     def forward(self, h, pending, ctx, cache):
         """Runs the layer on the residual stream h (fp32 [T,d]); ``pending`` are up to two
         increments not yet added to h.  Returns the new pending increments."""

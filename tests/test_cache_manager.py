@@ -257,6 +257,20 @@ def test_a_chunked_group_gets_no_more_pages_than_its_requests_can_hold():
     assert [small.total_pages(g) for g in range(2)] == [8, 8]
 
 
+def test_keys_and_values_of_widths_of_their_own():
+    # a mixer whose values are wider than its keys: the pool's halves are sized apart, and such a
+    # need shares no group with one of equal widths
+    needs = [CacheNeed(kv=KVNeed(2, 8, "full", 0, v_head_dim=24)), CacheNeed(kv=KVNeed(2, 8, "full")),
+             CacheNeed(kv=KVNeed(2, 8, "full", 0, v_head_dim=24))]
+    c = PagedCache(needs, 4, 6, 2, torch.float32, torch.device("cpu"))
+    assert c.n_groups() == 2 and c.group_of(0) == c.group_of(2) != c.group_of(1)
+    k, v = c.layer_pages(2)
+    assert tuple(k.shape) == (6, 2, 4, 8) and tuple(v.shape) == (6, 2, 24, 4)
+    k1, v1 = c.layer_pages(1)
+    assert tuple(k1.shape) == (6, 2, 4, 8) and tuple(v1.shape) == (6, 2, 8, 4)
+    assert not c.kv_tiled(0)
+
+
 def test_the_visibility_rules_have_one_definition():
     """The names and codes of the rules that say which keys a query reads come from one header;
     the cache manager (native) frees exactly what that header's rule no longer reads."""

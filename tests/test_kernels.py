@@ -415,8 +415,9 @@ class PagedKV:
             self.bt[s, b] = -1
 
 
-def attention_reference(kv, queries, qs, H, vis, span, softcap=0.0):
-    """queries: list of (request, position); qs [T,H,hd].  ``softcap``: the scaled scores are
+def attention_reference(kv, queries, qs, H, vis, span, softcap=0.0, slopes=None):
+    """queries: list of (request, position); qs [T,H,hd].  ``slopes`` ([H]): head h's scaled
+    score of the key at j gets slopes[h] * (j - p) added; ``softcap``: the scores are then
     capped, softcap * tanh(score / softcap), before the softmax."""
     out = torch.zeros(len(queries), H, kv.hd, dtype=torch.float64)
     for t, (s, p) in enumerate(queries):
@@ -425,21 +426,24 @@ def attention_reference(kv, queries, qs, H, vis, span, softcap=0.0):
             mask = plain.visible_mask(pos, vis, span)[p:p + 1]
         else:                        # the whole square would not fit: the query's own row of it
             mask = (pos >= plain_first(vis, span, p)).view(1, -1)
-        if not softcap:
+        if not softcap and slopes is None:
             out[t] = plain.attention(qs[t:t + 1].double(), kv.k[s][:p + 1].double(), kv.v[s][:p + 1].double(), mask)[0]
             continue
         k, v = kv.k[s][:p + 1].double(), kv.v[s][:p + 1].double()          # [keys, G, hd]
         for h in range(H):
             g = h // (H // k.shape[1])
             score = (k[:, g] @ qs[t, h].double()) / math.sqrt(kv.hd)
-            score = softcap * torch.tanh(score / softcap)
+            if slopes is not None:
+                score = score + float(slopes[h]) * (pos - p).double()
+            if softcap:
+                score = softcap * torch.tanh(score / softcap)
             score = score.masked_fill(~mask[0], float("-inf"))
             out[t, h] = torch.softmax(score, 0) @ v[:, g]
     return out
 
 
 def run_attention(kind, dtype, H, G, hd, ps, lens, queries, vis, span, n_splits=3, seed=0, planted=None, softcap=0.0,
-                  q_gain=1.0):
+                  q_gain=1.0, slopes=None):
     kv = PagedKV(lens, G, hd, ps, dtype, seed)
     T = len(queries)
     g = torch.Generator().manual_seed(seed + 1)
@@ -453,7 +457,8 @@ def run_attention(kind, dtype, H, G, hd, ps, lens, queries, vis, span, n_splits=
                                for s in range(len(lens))]):
         low = min([plain_first(vis, span, p) for ss, p in queries if ss == s], default=0)
         kv.drop_below(s, low)
-    ref = attention_reference(kv, queries, qs, H, vis, span, softcap)
+    ref = attention_reference(kv, queries, qs, H, vis, span, softcap, slopes)
+    sl = None if slopes is None else torch.tensor(slopes, dtype=torch.float32, device=DEV)
     positions = torch.tensor([p for _, p in queries], dtype=torch.int32, device=DEV)
     seq = torch.tensor([s for s, _ in queries], dtype=torch.int32, device=DEV)
     out = torch.zeros(T, H * hd, dtype=dtype, device=DEV)
@@ -462,12 +467,12 @@ def run_attention(kind, dtype, H, G, hd, ps, lens, queries, vis, span, n_splits=
     if kind != "generic":                        # the MFMA kernels read pages in operand order
         kp, vp = ops().kv_operand_order(kp, vp)
     if kind == "generic":
-        ops().attn_generic(q_dev, kp, vp, out, positions, seq, bt, T, H, G, hd, ps, vis, span, scale, softcap=softcap)
+        ops().attn_generic(q_dev, kp, vp, out, positions, seq, bt, T, H, G, hd, ps, vis, span, scale, softcap=softcap, slopes=sl)
         if ops().kv_tiled_ok(dtype, hd, ps):     # and the plain kernel reads them too, with the same bits
             again = torch.zeros_like(out)
             kpt, vpt = ops().kv_operand_order(kp, vp)
             ops().attn_generic(q_dev, kpt, vpt, again, positions, seq, bt, T, H, G, hd, ps, vis, span, scale, kv_tiled=True,
-                               softcap=softcap)
+                               softcap=softcap, slopes=sl)
             assert torch.equal(out, again)
     elif kind == "prefill":                      # runs of queries of one request are the portions
         runs = []
@@ -478,12 +483,12 @@ def run_attention(kind, dtype, H, G, hd, ps, lens, queries, vis, span, n_splits=
                 runs.append([s, 1])
         cu = torch.tensor([0] + list(np.cumsum([c for _, c in runs])), dtype=torch.int32, device=DEV)
         ops().attn_prefill(q_dev, kp, vp, out, positions, cu, [c for _, c in runs],
-                           bt[[s for s, _ in runs]].contiguous(), H, G, hd, ps, vis, span, scale, softcap=softcap)
+                           bt[[s for s, _ in runs]].contiguous(), H, G, hd, ps, vis, span, scale, softcap=softcap, slopes=sl)
     else:
         wsz = ops().attn_decode_workspace(T, H, hd, n_splits)
         scratch = torch.empty(wsz // 4, dtype=torch.float32, device=DEV)
         ops().attn_decode(q_dev, kp, vp, out, scratch, positions, seq, bt, T, H, G, hd, ps, vis, span, scale, n_splits,
-                          softcap=softcap)
+                          softcap=softcap, slopes=sl)
     got = out.double().cpu().view(T, H, hd)
     err = (got - ref).abs().max()
     assert torch.isfinite(got).all()
@@ -604,6 +609,29 @@ def test_attention_with_capped_scores(kind, dtype):
     qs = (torch.randn(len(queries), H, hd, generator=g) * 3.0).to(dtype)
     other = attention_reference(kv, queries, qs, H, "chunk", 128)
     assert (other - ref).abs().max() > 0.1
+
+
+@pytest.mark.parametrize("softcap", [0.0, 3.0])
+@pytest.mark.parametrize("kind,dtype", [("generic", torch.float32), ("generic", torch.bfloat16), ("decode", torch.bfloat16),
+                                        ("prefill", torch.bfloat16)])
+def test_attention_with_score_slopes(kind, dtype, softcap):
+    """A bias slope * (key - query position) per head on the scaled scores (an option of every
+    attention kernel), alone and before a cap: steep on some heads (they read their last few
+    keys), flat on others, zero on one."""
+    H, G, hd, ps = (8, 2, 128, 64) if kind != "generic" else (6, 3, 24, 8)
+    slopes = [0.0, 0.004, 0.03, 0.25, 1.0, 0.5, 0.06, 0.008][:H]
+    queries = [(0, p) for p in range(230, 300)] if kind == "prefill" else [(0, 299), (1, 128), (0, 40)]
+    if kind == "prefill":
+        queries += [(1, p) for p in range(0, 129)]
+    else:
+        queries = sorted(queries)
+    got, ref = run_attention(kind, dtype, H, G, hd, ps, [300, 129], queries, "full", 0, softcap=softcap, slopes=slopes)
+    kv = PagedKV([300, 129], G, hd, ps, dtype, 0)
+    g = torch.Generator().manual_seed(1)
+    qs = torch.randn(len(queries), H, hd, generator=g).to(dtype)
+    other = attention_reference(kv, queries, qs, H, "full", 0, softcap)
+    assert (other[:, 1:] - ref[:, 1:]).abs().max() > 0.1          # the slopes matter ...
+    assert (other[:, 0] - ref[:, 0]).abs().max() < 1e-12          # ... and a slope of zero changes nothing
 
 
 def test_prefill_attention_finds_one_far_key_among_thousands():

@@ -69,7 +69,8 @@ def poison_what_nobody_holds(eng, value=float("nan")):
     for g, group in enumerate(eng.cache.groups):
         free = sorted(set(range(group.n_pages)) - held_pages(eng, g))
         if free:
-            group.kv[:, :, torch.tensor(free, device=group.kv.device)] = value
+            for half in group.halves():
+                half[:, torch.tensor(free, device=half.device)] = value
 
 
 def run(eng, steps, after_step=None):

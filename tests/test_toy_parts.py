@@ -427,3 +427,66 @@ def test_attention_with_a_weighted_head_norm_before_a_rotation_of_part_of_the_he
     # the test has teeth: the other order of norm and rotation is another function
     q2 = plain.rms_norm(rotate((n @ W["b1.attn.q_proj"].T).view(T, HEADS, HD)), W["b1.attn.q_norm"], 1e-6)
     assert (q2 - q).abs().max() > 0.05
+
+
+@pytest.mark.parametrize("dtype,hd,page", [("float32", HD, 4), ("bfloat16", 64, 32)])
+def test_a_position_encoding_that_works_on_the_scores(dtype, hd, page):
+    """A position encoding of another kind, defined here: nothing rotates; head h's score of the key
+    at j for the query at p gets slope_h * (j - p) added.  The part hands the slopes to the built-in
+    mixer (`score_slopes`), whose kernels take them as an option: the plain kernel (32-bit, head size
+    8) and the MFMA kernels (bfloat16, head size 64: portions through the tiled kernel, single tokens
+    through the split one)."""
+    from spite_amd import Engine
+    from spite_amd.parts import PartSpec, BlockSpec, LayerCall, ModelSpec, PositionEncoding, register
+    import plain_llama4 as plain
+
+    @register("position", "toy_linear_bias")
+    class LinearBias(PositionEncoding):
+        def __init__(self, env, ratio):
+            self.env, self.ratio = env, float(ratio)
+
+        def score_slopes(self, n_heads):
+            return torch.tensor([self.ratio ** (h + 1) for h in range(n_heads)], dtype=torch.float32, device=self.env.device)
+
+    d = HEADS * hd
+    rms = lambda name: PartSpec("rms", {"width": d, "eps": 1e-5}, {"weight": name})
+    attn = PartSpec("attention", dict(hidden_size=d, n_heads=HEADS, n_kv_heads=KV, head_dim=hd,
+                                      position=PartSpec("toy_linear_bias", {"ratio": 0.4})),
+                    {k: f"attn.{k}" for k in ("q_proj", "k_proj", "v_proj", "o_proj")})
+    dense = PartSpec("dense_glu", {"hidden_size": d, "intermediate_size": 2 * d},
+                     {k: f"ffn.{k}" for k in ("gate_proj", "up_proj", "down_proj")})
+    sp = ModelSpec("ToyLinearBias", V, d, [BlockSpec("prenorm", rms("n1"), attn, rms("n2"), dense)], [LayerCall(0, 0)],
+                   rms("final"), "embed", "head")
+    g = torch.Generator().manual_seed(13)
+    rnd = lambda *s, std=0.2: torch.randn(*s, generator=g) * std
+    t = {"embed": rnd(V, d, std=1.0), "head": rnd(V, d), "final": 1 + rnd(d), "n1": 1 + rnd(d), "n2": 1 + rnd(d),
+         "attn.q_proj": rnd(HEADS * hd, d), "attn.k_proj": rnd(KV * hd, d), "attn.v_proj": rnd(KV * hd, d),
+         "attn.o_proj": rnd(d, HEADS * hd), "ffn.gate_proj": rnd(2 * d, d), "ffn.up_proj": rnd(2 * d, d), "ffn.down_proj": rnd(d, 2 * d)}
+    if dtype == "bfloat16":
+        t = {k: (v if k in ("final", "n1", "n2") else v.to(torch.bfloat16)) for k, v in t.items()}
+    W = {k: v.double() for k, v in t.items()}
+    toks = H.random_tokens(V, 75, 8)
+    T, pos = len(toks), torch.arange(len(toks))
+    h = W["embed"][torch.tensor(toks)]
+    n = plain.rms_norm(h, W["n1"], 1e-5)
+    q = (n @ W["attn.q_proj"].T).view(T, HEADS, hd)
+    k = (n @ W["attn.k_proj"].T).view(T, KV, hd)
+    v = (n @ W["attn.v_proj"].T).view(T, KV, hd)
+    mask, att = plain.visible_mask(pos, "full", 0), torch.zeros(T, HEADS, hd, dtype=torch.float64)
+    for hh in range(HEADS):
+        score = q[:, hh] @ k[:, hh // (HEADS // KV)].T / hd ** 0.5
+        score = score + 0.4 ** (hh + 1) * (pos[None, :] - pos[:, None]).double()
+        att[:, hh] = torch.softmax(score.masked_fill(~mask, float("-inf")), -1) @ v[:, hh // (HEADS // KV)]
+    assert (att - plain.attention(q, k, v, mask)).abs().max() > 0.02          # the bias matters here
+    h = h + att.reshape(T, HEADS * hd) @ W["attn.o_proj"].T
+    h = h + plain.swiglu_mlp(plain.rms_norm(h, W["n2"], 1e-5), W["ffn.gate_proj"], W["ffn.up_proj"], W["ffn.down_proj"])
+    ref = (plain.rms_norm(h, W["final"], 1e-5) @ W["head"].T).float().numpy()
+    reqs = {"x": toks}
+    eng = Engine(spec=sp, tensors={k: v.to("cuda:0") for k, v in t.items()}, dtype=dtype, page_size=page, cache_tokens=128,
+                 max_requests=2)
+    assert eng.slow_paths == {}
+    tol = 1e-4 if dtype == "float32" else 0.04 * float(abs(ref).max())
+    for steps in (H.schedule_whole(reqs), H.schedule_tail_one_by_one(reqs, tail=20), H.schedule_portions(reqs)):
+        got = H.collect(steps, H.run_trace_inprocess(eng, steps), V)
+        err = max(abs(got[("x", i)] - ref[i]).max() for i in range(T))
+        assert err < tol, (err, tol)
