@@ -699,6 +699,20 @@ extern "C" int spite_convert(const void* in, int in_dtype, void* out, int out_dt
     return 0;
 }
 
+// h[i] += d[i] over rows of width `d_cols` (fp32): an increment of the residual stream that no
+// norm's two addends have room for.  Row r of d is row r of h.
+__global__ void add_into_kernel(float* __restrict__ h, const float* __restrict__ d, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        h[i] += d[i];
+}
+extern "C" int spite_add_into(float* h, const float* d, size_t n, hipStream_t st) {
+    if (n == 0) return 0;
+    const int grid = (int)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
+    add_into_kernel<<<grid, 256, 0, st>>>(h, d, n);
+    SP_LAUNCH_CHECK("add_into");
+    return 0;
+}
+
 // ------------------------------------------------------------------ random weights
 // out[i] = mean + std * z(seed, key, i), z standard normal: element i of a tensor depends on the
 // seed, the tensor's key (a hash of its name) and i alone, not on the order in which tensors

@@ -39,6 +39,7 @@ def lib():
             "spite_router_top1": [P, P, P, P, P, I, I, I, P],
             "spite_moe_plan": [P, P, P, P, P, P, P, I, I, I, P],
             "spite_convert": [P, I, P, I, c_size_t, P],
+            "spite_add_into": [P, P, c_size_t, P],
             "spite_randn_fill": [P, I, c_size_t, ctypes.c_ulonglong, ctypes.c_ulonglong, F, F, P],
             "spite_gemm_generic": [P, I, P, L, I, P, I, I, I, I, I, P, I, P, P, P, I, P],
             "spite_attn_generic": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, F, P, I, P],
@@ -227,6 +228,14 @@ def convert(src, dst):
         raise KernelError("convert: sizes differ")
     _check(lib().spite_convert(_ptr(src, "src"), dtype_code(src.dtype), _ptr(dst, "dst"), dtype_code(dst.dtype),
                                src.numel(), _stream()), "convert")
+
+
+def add_into(h, d):
+    """h += d, both fp32 and of one size (an increment of the residual stream beyond the two
+    that a norm adds itself)."""
+    if h.numel() != d.numel() or not h.is_contiguous() or not d.is_contiguous():
+        raise KernelError(f"add_into: {tuple(h.shape)} and {tuple(d.shape)} must be contiguous and of one size")
+    _check(lib().spite_add_into(_ptr(h, "h", torch.float32), _ptr(d, "d", torch.float32), h.numel(), _stream()), "add_into")
 
 
 def randn_fill(t, seed: int, key: int, mean: float = 0.0, std: float = 1.0):

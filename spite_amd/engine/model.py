@@ -132,10 +132,9 @@ class Model:
                 if ctx.n_out == 0:
                     state["logits"] = torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.env.device)
                     continue
-                pending = state["pending"]
+                d1, d2 = P.two_increments(state["h"], state["pending"])
                 rows = ctx.ws.take((ctx.n_out, d), self.env.dtype)
-                self.final_norm.forward(state["h"], rows, d1=pending[0] if len(pending) > 0 else None,
-                                        d2=pending[1] if len(pending) > 1 else None, rows=ctx.logit_rows, write_h=False)
+                self.final_norm.forward(state["h"], rows, d1=d1, d2=d2, rows=ctx.logit_rows, write_h=False)
                 state["logits"] = step_ws.take((ctx.n_out, self.spec.vocab_size), torch.float32)
                 self.head.forward(rows, state["logits"], ctx)
         return state

@@ -198,6 +198,17 @@ class Head(Part):
         raise NotImplementedError
 
 
+def two_increments(h, pending):
+    """A norm adds up to two increments to the residual stream itself; what ``pending`` holds beyond
+    two (a feed-forward with three or more results a token, each written by a grouped product
+    to rows of its own) is added to ``h`` here first, in order.  Returns the two for the norm."""
+    if len(pending) > 2:
+        from ..csrc import hipops
+        for d in pending[2:]:
+            hipops.add_into(h, d[:h.shape[0]])
+    return (pending[0] if len(pending) > 0 else None, pending[1] if len(pending) > 1 else None)
+
+
 class Block(Part):
     def cache_needs(self) -> Dict[str, CacheNeed]:
         """What the block's parts ask of the cache manager, by names of the block's own choosing.
@@ -208,8 +219,8 @@ class Block(Part):
         return {"": self.mixer.cache_need()}
 
     def forward(self, h, pending, ctx, cache):
-        """Runs the layer on the residual stream h (fp32 [T,d]); ``pending`` are up to two
-        increments not yet added to h.  Returns the new pending increments."""
+        """Runs the layer on the residual stream h (fp32 [T,d]); ``pending`` are the increments
+        not yet added to h (see ``two_increments``).  Returns the new pending increments."""
         raise NotImplementedError
 
     def stages(self):

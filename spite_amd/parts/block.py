@@ -6,7 +6,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import Block, register, build as build_part
+from .base import Block, register, build as build_part, two_increments
 
 
 @register("block", "prenorm")
@@ -37,9 +37,8 @@ class PreNormBlock(Block):
                 (self.norm2.graph_safe and self.ffn.graph_safe, self._stage_ffn)]
 
     def _stage_norm1(self, state, ctx, cache):
-        h, pending = state["h"], state["pending"]
-        d1 = pending[0] if len(pending) > 0 else None
-        d2 = pending[1] if len(pending) > 1 else None
+        h = state["h"]
+        d1, d2 = two_increments(h, state["pending"])
         n = ctx.ws.take(tuple(h.shape), self.env.dtype)
         self.norm1.forward(h, n, d1=d1, d2=d2)
         state["normed"] = n

@@ -490,3 +490,90 @@ def test_a_position_encoding_that_works_on_the_scores(dtype, hd, page):
         got = H.collect(steps, H.run_trace_inprocess(eng, steps), V)
         err = max(abs(got[("x", i)] - ref[i]).max() for i in range(T))
         assert err < tol, (err, tol)
+
+
+def test_a_feed_forward_with_three_results_a_token():
+    """Every token goes to all three experts, the experts' outputs weighted by a softmax over the
+    router's logits: three increments of the residual stream come back from one feed-forward, one
+    more than a norm adds itself.  The framework adds the third to the stream before the next norm
+    (after the last layer too, before the final norm); the model has two such layers."""
+    from spite_amd import Engine
+    from spite_amd.parts import FeedForward, ParamSpec, register, PartSpec, BlockSpec, LayerCall, ModelSpec
+    from spite_amd.parts.linear import linear, Weight
+    import plain_llama4 as plain
+    n_exp, width = 3, 20
+
+    @register("ffn", "toy_all_three")
+    class AllThree(FeedForward):
+        wants_f32_input = True
+
+        def __init__(self, env, hidden_size, intermediate_size):
+            self.d, self.F = hidden_size, intermediate_size
+
+        def params(self):
+            return {"router": ParamSpec((n_exp, self.d), kind="vector"),
+                    "gate_up": ParamSpec((n_exp, 2 * self.F, self.d)), "down": ParamSpec((n_exp, self.d, self.F))}
+
+        def load(self, t):
+            self.router, self.w_gate_up, self.w_down = t["router"], Weight(t["gate_up"]), Weight(t["down"])
+
+        def forward(self, x, x32, ctx, projected=None):
+            T = x.shape[0]
+            weight = torch.softmax(x32[:T] @ self.router.T, dim=-1)               # [T, 3]
+            dev = x.device
+            offsets = (torch.arange(n_exp + 1, device=dev) * T).to(torch.int32)   # group e: slots [eT, (e+1)T)
+            src = torch.arange(T, device=dev, dtype=torch.int32).repeat(n_exp)
+            rows = torch.arange(n_exp * T, device=dev, dtype=torch.int32)         # slot s writes row s
+            scale = weight.T.contiguous().view(-1).float()
+            act = ctx.ws.take((n_exp * T, self.F), x.dtype)
+            linear(x, self.w_gate_up, act, glu=True, offsets=offsets, n_groups=n_exp, a_rows=src, rows=n_exp * T, max_rows=T)
+            y = ctx.ws.take((n_exp * T, self.d), torch.float32)
+            linear(act, self.w_down, y, offsets=offsets, n_groups=n_exp, a_scale=scale, y_rows=rows, rows=n_exp * T, max_rows=T)
+            return tuple(y[e * T:(e + 1) * T] for e in range(n_exp))
+
+    rms = lambda name: PartSpec("rms", {"width": D, "eps": 1e-5}, {"weight": name})
+    blocks = []
+    for b in range(2):
+        attn = PartSpec("attention", dict(hidden_size=D, n_heads=HEADS, n_kv_heads=KV, head_dim=HD,
+                                          position=PartSpec("rotary", {"head_dim": HD, "theta": 100.0})),
+                        {k: f"b{b}.attn.{k}" for k in ("q_proj", "k_proj", "v_proj", "o_proj")})
+        ffn = PartSpec("toy_all_three", {"hidden_size": D, "intermediate_size": width},
+                       {k: f"b{b}.ffn.{k}" for k in ("router", "gate_up", "down")})
+        blocks.append(BlockSpec("prenorm", rms(f"b{b}.n1"), attn, rms(f"b{b}.n2"), ffn))
+    spec3 = ModelSpec("ToyThree", V, D, blocks, [LayerCall(0, 0), LayerCall(1, 1)], rms("final"), "embed", "head")
+    g = torch.Generator().manual_seed(5)
+    r = lambda *s: torch.randn(*s, generator=g) * 0.3
+    t = {"embed": r(V, D), "head": r(V, D), "final": 1 + r(D) * 0.1}
+    for b in range(2):
+        t[f"b{b}.n1"], t[f"b{b}.n2"] = 1 + r(D) * 0.1, 1 + r(D) * 0.1
+        t[f"b{b}.attn.q_proj"], t[f"b{b}.attn.o_proj"] = r(HEADS * HD, D), r(D, HEADS * HD)
+        t[f"b{b}.attn.k_proj"], t[f"b{b}.attn.v_proj"] = r(KV * HD, D), r(KV * HD, D)
+        t[f"b{b}.ffn.router"], t[f"b{b}.ffn.gate_up"], t[f"b{b}.ffn.down"] = r(n_exp, D) * 2, r(n_exp, 2 * width, D), r(n_exp, D, width)
+
+    def plain_three(tokens):
+        W = {k: v.double() for k, v in t.items()}
+        T = len(tokens)
+        pos = torch.arange(T)
+        h = W["embed"][torch.tensor(tokens)]
+        inv = plain.rope_inv_freq(HD, 100.0, None)
+        for b in range(2):
+            n = plain.rms_norm(h, W[f"b{b}.n1"], 1e-5)
+            q = plain.apply_rope((n @ W[f"b{b}.attn.q_proj"].T).view(T, HEADS, HD), pos, inv)
+            k = plain.apply_rope((n @ W[f"b{b}.attn.k_proj"].T).view(T, KV, HD), pos, inv)
+            v = (n @ W[f"b{b}.attn.v_proj"].T).view(T, KV, HD)
+            h = h + plain.attention(q, k, v, plain.visible_mask(pos, "full", 0)).reshape(T, HEADS * HD) @ W[f"b{b}.attn.o_proj"].T
+            n = plain.rms_norm(h, W[f"b{b}.n2"], 1e-5)
+            wt = torch.softmax(n @ W[f"b{b}.ffn.router"].T, dim=-1)
+            for e in range(n_exp):
+                gu = n @ W[f"b{b}.ffn.gate_up"][e].T
+                h = h + wt[:, e:e + 1] * ((F.silu(gu[:, :width]) * gu[:, width:]) @ W[f"b{b}.ffn.down"][e].T)
+        return (plain.rms_norm(h, W["final"], 1e-5) @ W["head"].T).float().numpy()
+
+    eng = Engine(spec=spec3, tensors=t, dtype="float32", page_size=4, cache_tokens=96, max_requests=3)
+    reqs = {"x": H.random_tokens(V, 21, 1), "y": H.random_tokens(V, 10, 2)}
+    ref = {(rid, i): row for rid, toks in reqs.items() for i, row in enumerate(plain_three(toks))}
+    # the third expert's share is no rounding matter: without it the logits are far off
+    for steps in (H.schedule_whole(reqs), H.schedule_tail_one_by_one(reqs, tail=6), H.schedule_portions(reqs, sizes=(3, 2, 5))):
+        got = H.collect(steps, H.run_trace_inprocess(eng, steps), V)
+        d, where = H.max_diff(got, ref)
+        assert d < 1e-4, (d, where)
