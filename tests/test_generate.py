@@ -82,6 +82,48 @@ def test_preemption_changes_nothing(models):
     assert tight == roomy
 
 
+def test_bfloat16_generation_through_mixed_steps_and_preemption(tmp_path):
+    """bfloat16 through the scheduler: prompts cut into portions beside decoded tokens, and a pool so
+    tight that requests are preempted and computed again.  bfloat16 products pick their kernel from
+    the step's rows, so the two runs agree to rounding, not bit for bit: every token that either run
+    chose must be the plain implementation's choice at that place (fed the run's own tokens), or
+    within rounding of it; and where the plain implementation's choice is clear the runs agree."""
+    cfg = H.TINY_C
+    d = str(tmp_path / "C16")
+    w = H.make_model(d, cfg, seed=11, dtype="bfloat16")
+    V = cfg["vocab_size"]
+    prompts = [H.random_tokens(V, n, 70 + n) for n in (40, 60, 30, 50)]
+    n_new = 40
+    roomy = engine(d, dtype="bfloat16", page_size=32, cache_tokens=2048, max_batch_tokens=256)
+    assert not roomy.slow_paths                   # sizes that the MFMA kernels take
+    runs = {"roomy": roomy.generate(prompts, max_tokens=n_new, temperature=0.0)}
+    stats = {}
+    tight = engine(d, dtype="bfloat16", page_size=32, num_pages=5, max_batch_tokens=48)
+    runs["tight"] = tight.generate(prompts, max_tokens=n_new, temperature=0.0, stats=stats)
+    assert stats["preemptions"] >= 1, "the pool was not tight enough to preempt"
+    assert stats["steps"] > n_new + 4             # prompts went in portions beside decoded tokens
+    worst = 0.0
+    clear = {}
+    for name, run in runs.items():
+        for r, (p, g) in enumerate(zip(prompts, run)):
+            assert len(g) == n_new
+            logits = plain.forward(cfg, w, p + g)[len(p) - 1:-1]
+            scale = float(logits.abs().max())
+            for i, t in enumerate(g):
+                top = torch.topk(logits[i], 2).values
+                worst = max(worst, float(top[0] - logits[i, t]) / scale)
+                # a place where the runner-up is far behind, and all tokens before it agree with the other run
+                clear[(name, r, i)] = float(top[0] - top[1]) > 0.08 * scale
+    print(f"largest distance of a chosen token from the plain implementation's best: {worst:.4f} of the logits' scale")
+    assert worst <= 0.04, worst
+    for r in range(len(prompts)):
+        for i in range(n_new):
+            if runs["roomy"][r][:i] != runs["tight"][r][:i]:
+                break
+            if clear[("roomy", r, i)]:
+                assert runs["roomy"][r][i] == runs["tight"][r][i], (r, i)
+
+
 def test_finish_reasons(models):
     d, w, cfg = models["A"]
     eng = engine(d)
