@@ -170,6 +170,10 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
             __builtin_amdgcn_sched_group_barrier(0x100, NS, 0);
             __builtin_amdgcn_sched_group_barrier(0x008, NS, 0);
         }
+        // (nothing of what follows moves up between them: the reads of V^T below would otherwise be
+        // counted among the eight reads above, and the K operands they displace be read one by one,
+        // each product waiting for its own)
+        __builtin_amdgcn_sched_barrier(0);
         // on the cheap path the run's V^T operands are asked for before the softmax, whose arithmetic
         // hides their way
         bf16x8 vf[NDT][2];
