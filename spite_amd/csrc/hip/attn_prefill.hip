@@ -304,16 +304,21 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
     }
+    if (i < i_end && pq_max >= 0) {
+        // every query of the tile reads the keys of the steps that follow: a page that is missing
+        // poisons them all.  The pages are looked up here, 64 at a time, not run by run in the loop
+        // (a table entry per run is a scalar load that the next run's reads of LDS would wait for).
+        const int k_lo = (uA + (i - n_edge)) * PF_KEYS, k_hi = (uA + (i_end - n_edge)) * PF_KEYS;
+        bool bad = false;
+        for (int pg = k_lo / ps + lane; pg <= (k_hi - 1) / ps; pg += 64) bad |= pg >= max_blocks || bt[pg] < 0;
+        poison = __any(bad);
+    }
     for (; i < i_end; ++i, buf ^= 1) {
         const int u = uA + (i - n_edge);
         if (i + 1 < i_end) stage(u + 1, buf ^ 1);
         if (pq_max >= 0) {
 #pragma unroll
-            for (int h = 0; h < PF_RUNS; ++h) {
-                // every query of the tile reads these keys: a page that is missing poisons them all
-                poison |= page_of(u * PF_KEYS + h * 32) < 0;
-                run32(u * PF_KEYS + h * 32, buf * STEP + h * RUN, std::false_type{});
-            }
+            for (int h = 0; h < PF_RUNS; ++h) run32(u * PF_KEYS + h * 32, buf * STEP + h * RUN, std::false_type{});
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
